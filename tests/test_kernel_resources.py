@@ -13,7 +13,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 sys.path.insert(0, os.path.join(ROOT, "tools"))
 
 pytestmark = pytest.mark.skipif(not os.path.exists("/opt/rocm/lib/llvm/bin/llvm-readelf"),
-                                reason="needs the ROCm LLVM binutils (llvm-readelf / llvm-objdump)")
+                                reason="needs the ROCm LLVM binutils (llvm-readelf)")
 
 
 @pytest.fixture(scope="module")
@@ -90,29 +90,6 @@ def test_norm_and_sampler_kernels_stay_small(kernels):
             assert r["vgpr_count"] <= 128, (r["name"], r["vgpr_count"])
     for r in _named(kernels, "add_rmsnorm_splitk_kernel"):
         assert r["vgpr_count"] <= 160, (r["name"], r["vgpr_count"])
-
-
-def test_prefill_kernel_isa_has_none_of_the_patterns_this_project_removed():
-    """Disassembly of the built prefill attention kernels. Each bound below is a pattern hipcc once put into this
-    kernel's tile loop and that cost 3-12 % until it was found by reading the .s ("Prefill attention"):
-      * a readfirstlane "waterfall" loop around every K/V buffer load (tile coordinates no longer provably uniform):
-        s_cbranch_execnz loops and v_readfirstlane counts jump;
-      * 49 register moves zero-filling the score tile at every loop head: v_mov_b32 count jumps by ~100 (2 unrolled tiles);
-      * an LDS round trip (ds_bpermute) in the per-tile softmax chain: only the two prologue scans may use it;
-      * 16 dwordx2 epilogue stores instead of 8 dwordx4; AGPRs used as spill slots (v_accvgpr copies)."""
-    from nano_vllm_amd import build
-    import kernel_resources
-    import re
-    dis = kernel_resources.disassemble(build.build(), "prefill_attn_kernel")
-    assert len(dis) == 6, sorted(dis)        # {paged, paged fp8, packed} x {4 waves, 8 waves}
-    for name, text in dis.items():
-        assert text.count("v_mfma_f32_32x32x16_bf16") == 64, name          # two unrolled tiles x 32 MFMAs, nothing else
-        assert text.count("s_cbranch_execnz") <= 2, (name, "waterfall loops")
-        assert text.count("v_readfirstlane_b32") <= 16, (name, "waterfall loops")
-        assert len(re.findall(r"\bv_mov_b32", text)) <= 80, (name, "zero fill of the score registers")
-        assert text.count("ds_bpermute_b32") <= 12, (name, "LDS round trip in the tile loop")
-        assert text.count("v_accvgpr") == 0 and "scratch_" not in text, (name, "spill copies")
-        assert len(re.findall(r"_store_dwordx4", text)) == 8 and not re.findall(r"_store_dwordx2", text), name
 
 
 def test_generated_prefill_loop_owns_its_register_file(kernels):

@@ -78,33 +78,6 @@ def kernels(path: str) -> list[dict]:
     return rows
 
 
-def disassemble(path: str, fragment: str) -> dict[str, str]:
-    """{kernel symbol: disassembly text} of every kernel of the library whose (mangled) name contains `fragment`."""
-    out = {}
-    for co in code_objects(path):
-        with tempfile.NamedTemporaryFile(suffix=".co") as tf:
-            tf.write(co)
-            tf.flush()
-            syms = subprocess.run([f"{LLVM}/llvm-readelf", "-s", "-W", tf.name], capture_output=True, text=True).stdout
-            names = sorted({ln.split()[-1] for ln in syms.splitlines()
-                            if " FUNC " in ln and fragment in ln and not ln.split()[-1].endswith(".kd")})
-            if not names:
-                continue
-            text = subprocess.run([f"{LLVM}/llvm-objdump", "-d", "--no-show-raw-insn", "--mcpu=gfx950",
-                                   "--disassemble-symbols=" + ",".join(names), tf.name],
-                                  capture_output=True, text=True).stdout
-        cur = None
-        for ln in text.splitlines():
-            m = re.match(r"^[0-9a-f]+ <([^>]+)>:", ln)
-            if m:
-                cur = m.group(1) if m.group(1) in names else None
-                if cur:
-                    out[cur] = ""
-            elif cur:
-                out[cur] += ln + "\n"
-    return out
-
-
 if __name__ == "__main__":
     lib = next((a for a in sys.argv[1:] if not a.startswith("--")),
                os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "nano_vllm_amd", "lib",
