@@ -45,14 +45,26 @@ class Config:
     seed: int = 0
     dummy_weights: bool = False
     kv_cache_dtype: str = "bf16"         # "fp8": OCP e4m3 KV cache (halves decode bytes; outside the reference's numerics)
+    dtype: str = "auto"                  # activation / weight type: "auto" (the checkpoint's, bfloat16 if it names none),
+    #                                      "bfloat16", or "float32" for families whose kernels exist in 32-bit (registry.ModelSpec.dtypes)
 
     def __post_init__(self):
         assert os.path.isdir(self.model), f"model directory not found: {self.model}"
-        assert self.kvcache_block_size % 256 == 0
         assert 1 <= self.tensor_parallel_size <= 8
+        from .registry import resolve, spec_of
         if self.hf_config is None:
-            from transformers import AutoConfig
-            self.hf_config = AutoConfig.from_pretrained(self.model)
+            spec, self.hf_config = resolve(self.model)
+        else:
+            spec = spec_of(self.hf_config)
+        # page sizes the family's attention kernels take (the paged-KV transformer kernels: 256-token pages)
+        assert self.kvcache_block_size % spec.block_multiple == 0, \
+            f"kvcache_block_size must be a multiple of {spec.block_multiple} for {spec.name}"
+        if self.dtype in ("bf16", "fp32"):
+            self.dtype = {"bf16": "bfloat16", "fp32": "float32"}[self.dtype]
+        assert self.dtype == "auto" or self.dtype in spec.dtypes, f"{spec.name} runs in {spec.dtypes}, not {self.dtype!r}"
+        if spec.stateful:
+            assert self.tensor_parallel_size == 1, f"{spec.name}: state slots are per process; tensor parallelism is not wired for it"
+            assert self.kv_cache_dtype == "bf16", "the fp8 KV cache belongs to the 128-wide paged-KV kernels"
         self.max_model_len = min(self.max_model_len, self.hf_config.max_position_embeddings)
         assert self.max_num_batched_tokens >= 1 and self.max_num_seqs >= 1
         assert self.kv_cache_dtype in ("bf16", "fp8"), "kv_cache_dtype must be 'bf16' or 'fp8'"

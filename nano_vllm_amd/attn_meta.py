@@ -6,13 +6,15 @@ the runner publishes per-step metadata with `set_context(...)`, `Attention.forwa
 names and the positional order of `set_context` follow the reference so reference-style
 callers work unchanged; four extra fields carry what the HIP decode kernel needs (its split-KV
 workspace, the static `max_context` bound that makes the launch hipGraph-safe, the per-step work
-plan shared by every layer's launch — ops.decode_plan — and whether that plan carries a shared prefix).
+plan shared by every layer's launch — ops.decode_plan — and whether that plan carries a shared prefix), and one carries
+the packed-portion description that stateful layers read (`portions`: ops_seq.Portions — per portion its token rows, the
+tokens earlier steps already processed and its state slot).
 """
 from __future__ import annotations
 
 _FIELDS = ("is_prefill", "cu_seqlens_q", "cu_seqlens_k", "max_seqlen_q", "max_seqlen_k", "slot_mapping",
-           "context_lens", "block_tables", "decode_workspace", "max_context", "decode_plan", "shared_prefix")
-_DEFAULTS = (False, None, None, 0, 0, None, None, None, None, 0, None, False)
+           "context_lens", "block_tables", "decode_workspace", "max_context", "decode_plan", "shared_prefix", "portions")
+_DEFAULTS = (False, None, None, 0, 0, None, None, None, None, 0, None, False, None)
 
 
 class Context:

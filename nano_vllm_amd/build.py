@@ -1,4 +1,6 @@
-"""Build libnvl_hip.so (the C-ABI HIP kernel library) for gfx950 with hipcc.
+"""Build the C-ABI HIP kernel libraries for gfx950 with hipcc: libnvl_hip.so (csrc/*.hip: the paged-KV transformer
+path) and libnvl_seq.so (csrc/seq/*.hip: stateful sequence mixers, windowed attention, 32-bit residual norms). Each is
+built on its own, so a model that needs one of them does not wait for the other.
 
 In-tree build: the .so lands in nano_vllm_amd/lib/ (git-ignored, shipped by gpurun).
 hipcc cross-compiles without a GPU, so this also runs in the CPU-only build container.
@@ -115,6 +117,67 @@ def build(force: bool = False, verbose: bool = False) -> str:
     return LIB
 
 
+# ---- libnvl_seq.so ------------------------------------------------------------------------------------------------
+SEQ_CSRC = os.path.join(CSRC, "seq")
+LIB_SEQ = os.path.join(LIBDIR, "libnvl_seq.so")
+# packed 32-bit float instructions are kept out of these kernels: their recurrences and norms are 32-bit throughout
+SEQ_FLAGS = FLAGS + ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+
+def seq_sources() -> list[str]:
+    return sorted(os.path.join(SEQ_CSRC, f) for f in os.listdir(SEQ_CSRC) if f.endswith(".hip"))
+
+
+def _seq_digest() -> str:
+    h = hashlib.sha256()
+    files = seq_sources() + [os.path.join(SEQ_CSRC, f) for f in sorted(os.listdir(SEQ_CSRC)) if f.endswith(".h")]
+    files.append(os.path.join(HERE, "..", "include", "nvl_seq.h"))
+    for f in files:
+        with open(f, "rb") as fh:
+            h.update(os.path.basename(f).encode())
+            h.update(fh.read())
+    h.update(" ".join(SEQ_FLAGS).encode())
+    return h.hexdigest()
+
+
+def build_seq(force: bool = False) -> str:
+    """Compile csrc/seq/*.hip into libnvl_seq.so (a few seconds per file, in parallel); returns its path."""
+    os.makedirs(LIBDIR, exist_ok=True)
+    stamp = os.path.join(LIBDIR, "libnvl_seq.stamp")
+    digest = _seq_digest()
+    if not force and os.path.exists(LIB_SEQ) and os.path.exists(stamp):
+        with open(stamp) as fh:
+            if fh.read().strip() == digest:
+                return LIB_SEQ
+    hipcc = _hipcc()
+    objdir = os.path.join(LIBDIR, "obj")
+    os.makedirs(objdir, exist_ok=True)
+    procs, objs = [], []
+    for src in seq_sources():
+        obj = os.path.join(objdir, "seq_" + os.path.basename(src)[:-4] + ".o")
+        objs.append(obj)
+        procs.append((src, subprocess.Popen([hipcc, f"--offload-arch={ARCH}", *SEQ_FLAGS, "-c", src, "-o", obj],
+                                            stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
+    failed = False
+    for src, p in procs:
+        out, _ = p.communicate()
+        if p.returncode != 0:
+            failed = True
+            sys.stderr.write(f"--- hipcc failed on {src}\n{out}\n")
+    if failed:
+        raise RuntimeError("hipcc compilation failed")
+    tmp = LIB_SEQ + f".{os.getpid()}.tmp"
+    subprocess.run([hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", *objs, "-o", tmp], check=True)
+    os.replace(tmp, LIB_SEQ)                     # (atomic: two processes may build a fresh checkout at once)
+    with open(stamp, "w") as fh:
+        fh.write(digest)
+    return LIB_SEQ
+
+
 if __name__ == "__main__":
-    path = build(force="--force" in sys.argv, verbose="--verbose" in sys.argv)
-    print(path)
+    if "--seq" in sys.argv:
+        print(build_seq(force="--force" in sys.argv))
+    else:
+        path = build(force="--force" in sys.argv, verbose="--verbose" in sys.argv)
+        print(path)
+        print(build_seq(force="--force" in sys.argv))

@@ -1,0 +1,154 @@
+// Residual-stream kernels: embedding + sinusoid, output-side scalar RMS norms with the residual add, the final norm on
+// selected rows, xIELU. The residual stream is 32-bit; a copy in the activation type feeds the next matrix product.
+#include "seq_common.h"
+#include <string.h>
+
+namespace {
+thread_local char g_err[512] = "";
+}
+void nvs_set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+}
+int nvs_check_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    nvs_set_error("%s: HIP launch failed: %s", what, hipGetErrorString(e));
+    return NVS_ELAUNCH;
+  }
+  return NVS_OK;
+}
+extern "C" int nvs_abi_version(void) { return 1; }
+extern "C" const char* nvs_last_error(void) { return g_err; }
+
+namespace {
+
+template <typename T>
+__global__ void embed_sinusoid_kernel(const T* __restrict__ table, const int64_t* __restrict__ ids, const int64_t* __restrict__ pos,
+                                      int width, float scale, float log2_base, float* __restrict__ x, T* __restrict__ xh) {
+  const int64_t t = blockIdx.x;
+  const int64_t id = ids[t];
+  const float p = (float)pos[t];
+  for (int c = threadIdx.x; c < width; c += blockDim.x) {
+    const int i = c >> 1;
+    // base^(-2i/width) in 32-bit; the angle is the product of two 32-bit numbers
+    const float inv = exp2f(-(2.f * (float)i / (float)width) * log2_base);
+    const float ang = p * inv;
+    const float pe = (c & 1) ? cosf(ang) : sinf(ang);
+    const float v = ldf(table + id * width + c) * scale + pe;
+    x[t * width + c] = v;
+    if (xh) stf(xh + t * width + c, v);
+  }
+}
+
+// one workgroup per token row
+template <typename T>
+__global__ void norm_residual_kernel(const T* __restrict__ m, const T* __restrict__ m2, const T* __restrict__ w1,
+                                     const T* __restrict__ w2, const T* __restrict__ g, int width, float eps,
+                                     float* __restrict__ x, T* __restrict__ xh) {
+  __shared__ float red[16];
+  const int64_t t = blockIdx.x;
+  const float gv = ldf(g);
+  float ss = 0.f;
+  if (m2 == nullptr) {
+    for (int c = threadIdx.x; c < width; c += blockDim.x) {
+      const float v = ldf(m + t * width + c);
+      ss += v * v;
+    }
+    const float r = rsqrtf(block_sum(ss, red) / (float)width + eps);
+    for (int c = threadIdx.x; c < width; c += blockDim.x) {
+      const float v = x[t * width + c] + gv * (ldf(m + t * width + c) * r);
+      x[t * width + c] = v;
+      if (xh) stf(xh + t * width + c, v);
+    }
+    return;
+  }
+  float s2 = 0.f;
+  for (int c = threadIdx.x; c < width; c += blockDim.x) {
+    const float a = ldf(m + t * width + c), b = ldf(m2 + t * width + c);
+    ss += a * a;
+    s2 += b * b;
+  }
+  const float r1 = rsqrtf(block_sum(ss, red) / (float)width + eps);
+  const float r2 = rsqrtf(block_sum(s2, red) / (float)width + eps);
+  float s3 = 0.f;
+  for (int c = threadIdx.x; c < width; c += blockDim.x) {
+    const float v = 0.5f * (ldf(m + t * width + c) * r1 * ldf(w1 + c) + ldf(m2 + t * width + c) * r2 * ldf(w2 + c));
+    s3 += v * v;
+  }
+  const float r3 = rsqrtf(block_sum(s3, red) / (float)width + eps);
+  for (int c = threadIdx.x; c < width; c += blockDim.x) {
+    const float mm = 0.5f * (ldf(m + t * width + c) * r1 * ldf(w1 + c) + ldf(m2 + t * width + c) * r2 * ldf(w2 + c));
+    const float v = x[t * width + c] + gv * (mm * r3);
+    x[t * width + c] = v;
+    if (xh) stf(xh + t * width + c, v);
+  }
+}
+
+template <typename T>
+__global__ void scalar_norm_rows_kernel(const float* __restrict__ x, const int32_t* __restrict__ rows, int width,
+                                        const T* __restrict__ g, float eps, T* __restrict__ out) {
+  __shared__ float red[16];
+  const int64_t r = blockIdx.x;
+  const int64_t src = rows ? (int64_t)rows[r] : r;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < width; c += blockDim.x) {
+    const float v = x[src * width + c];
+    ss += v * v;
+  }
+  const float k = rsqrtf(block_sum(ss, red) / (float)width + eps) * ldf(g);
+  for (int c = threadIdx.x; c < width; c += blockDim.x) stf(out + r * width + c, x[src * width + c] * k);
+}
+
+template <typename T>
+__global__ void xielu_kernel(const T* __restrict__ in, const T* __restrict__ pq, float beta, int64_t numel, T* __restrict__ out) {
+  const float ap = softplusf_(ldf(pq)), aq = beta + softplusf_(ldf(pq + 1));
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < numel; i += (int64_t)gridDim.x * blockDim.x) {
+    const float z = ldf(in + i);
+    const float v = z > 0.f ? ap * z * z + beta * z : aq * (expm1f(z) - z) + beta * z;
+    stf(out + i, v);
+  }
+}
+
+int threads_for(int width) { return width >= 1024 ? 256 : (width >= 256 ? 128 : 64); }
+
+}  // namespace
+
+extern "C" int nvs_embed_sinusoid(const void* table, int dtype, const int64_t* ids, const int64_t* pos, int64_t n, int width,
+                                  float scale, float base, float* x, void* xh, void* stream) {
+  NVS_REQUIRE(table && ids && pos && x && n >= 0 && width > 0 && base > 1.f, "nvs_embed_sinusoid: bad argument");
+  if (n == 0) return NVS_OK;
+  NVS_DISPATCH(dtype, embed_sinusoid_kernel<T><<<dim3((unsigned)n), dim3(threads_for(width)), 0, (hipStream_t)stream>>>(
+                          (const T*)table, ids, pos, width, scale, log2f(base), x, (T*)xh));
+  return nvs_check_launch("nvs_embed_sinusoid");
+}
+
+extern "C" int nvs_norm_residual(const void* m, const void* m2, const void* w1, const void* w2, const void* g, int dtype,
+                                 int64_t n, int width, float eps, float* x, void* xh, void* stream) {
+  NVS_REQUIRE(m && g && x && n >= 0 && width > 0, "nvs_norm_residual: bad argument");
+  NVS_REQUIRE(!m2 || (w1 && w2), "nvs_norm_residual: two branches need both channel weights");
+  if (n == 0) return NVS_OK;
+  NVS_DISPATCH(dtype, norm_residual_kernel<T><<<dim3((unsigned)n), dim3(threads_for(width)), 0, (hipStream_t)stream>>>(
+                          (const T*)m, (const T*)m2, (const T*)w1, (const T*)w2, (const T*)g, width, eps, x, (T*)xh));
+  return nvs_check_launch("nvs_norm_residual");
+}
+
+extern "C" int nvs_scalar_norm_rows(const float* x, const int32_t* rows, int64_t nrows, int width, const void* g, int dtype,
+                                    float eps, void* out, void* stream) {
+  NVS_REQUIRE(x && g && out && nrows >= 0 && width > 0, "nvs_scalar_norm_rows: bad argument");
+  if (nrows == 0) return NVS_OK;
+  NVS_DISPATCH(dtype, scalar_norm_rows_kernel<T><<<dim3((unsigned)nrows), dim3(threads_for(width)), 0, (hipStream_t)stream>>>(
+                          x, rows, width, (const T*)g, eps, (T*)out));
+  return nvs_check_launch("nvs_scalar_norm_rows");
+}
+
+extern "C" int nvs_xielu(const void* in, const void* pq, float beta, int dtype, int64_t numel, void* out, void* stream) {
+  NVS_REQUIRE(in && pq && out && numel >= 0, "nvs_xielu: bad argument");
+  if (numel == 0) return NVS_OK;
+  const int64_t blocks = (numel + 255) / 256;
+  NVS_DISPATCH(dtype, xielu_kernel<T><<<dim3((unsigned)(blocks > 65536 ? 65536 : blocks)), dim3(256), 0, (hipStream_t)stream>>>(
+                          (const T*)in, (const T*)pq, beta, numel, (T*)out));
+  return nvs_check_launch("nvs_xielu");
+}

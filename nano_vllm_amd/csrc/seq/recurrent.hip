@@ -1,0 +1,268 @@
+// Stateful sequence kernels: causal convolution, real-gated linear recurrence, state-space-duality recurrence (recurrent
+// form), gated group norm. State lives in 32-bit in per-sequence slots; a portion whose first token is position 0 starts
+// from zeros whatever the slot holds.
+#include "seq_common.h"
+
+namespace {
+
+constexpr int MAX_TAPS = 8;
+
+// ---- causal convolution -------------------------------------------------------------------------------------------
+// one thread per (token, channel); inputs before the portion come from the slot's tail (or are zero at a sequence start)
+template <typename T>
+__global__ void causal_conv_kernel(const T* __restrict__ in, int64_t in_stride, const T* __restrict__ w, const T* __restrict__ b,
+                                   int channels, int taps, int act, const int32_t* __restrict__ cu_q,
+                                   const int32_t* __restrict__ ctx0, const int32_t* __restrict__ slot,
+                                   const int32_t* __restrict__ tseq, const float* __restrict__ state, float* __restrict__ out,
+                                   int64_t t0) {
+  const int64_t t = t0 + blockIdx.y;
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= channels) return;
+  const int s = tseq[t];
+  const int64_t q0 = cu_q[s];
+  const int64_t rel = t - q0;                       // index inside the portion
+  const bool fresh = ctx0[s] == 0;
+  const float* tail = state + (int64_t)slot[s] * (taps - 1) * channels;
+  float acc = b ? ldf(b + c) : 0.f;
+  for (int j = 0; j < taps; ++j) {
+    const int64_t back = (taps - 1) - j;            // tokens before the current one
+    float v;
+    if (rel >= back) {
+      v = ldf(in + (t - back) * in_stride + c);
+    } else if (fresh) {
+      v = 0.f;
+    } else {
+      // tail[k] is the input (taps-1-k) tokens before the portion's first token; this tap looks (back - rel) before it
+      const int k = (taps - 1) - (int)(back - rel);
+      v = tail[(int64_t)k * channels + c];
+    }
+    acc += ldf(w + (int64_t)c * taps + j) * v;
+  }
+  if (act == 1) acc = siluf_(acc);
+  out[t * channels + c] = acc;
+}
+
+// one thread per (portion, channel): the new tail is read completely before it is written
+template <typename T>
+__global__ void conv_state_kernel(const T* __restrict__ in, int64_t in_stride, int channels, int taps,
+                                  const int32_t* __restrict__ cu_q, const int32_t* __restrict__ ctx0,
+                                  const int32_t* __restrict__ slot, float* __restrict__ state) {
+  const int s = blockIdx.y;
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= channels) return;
+  const int64_t q0 = cu_q[s], len = cu_q[s + 1] - q0;
+  if (len <= 0) return;
+  const bool fresh = ctx0[s] == 0;
+  float* tail = state + (int64_t)slot[s] * (taps - 1) * channels;
+  float nv[MAX_TAPS];
+  for (int k = 0; k < taps - 1; ++k) {
+    const int64_t back = (taps - 1) - k;            // new tail[k] = input `back` tokens before the END of the portion
+    float v;
+    if (len >= back) {
+      v = ldf(in + (q0 + len - back) * in_stride + c);
+    } else if (fresh) {
+      v = 0.f;
+    } else {
+      v = tail[(int64_t)(k + len) * channels + c];  // the old tail, shifted by the portion's length
+    }
+    nv[k] = v;
+  }
+  for (int k = 0; k < taps - 1; ++k) tail[(int64_t)k * channels + c] = nv[k];
+}
+
+// ---- real-gated linear recurrence ---------------------------------------------------------------------------------
+// one thread per (portion, channel), sequential over the portion's tokens; loads do not depend on the recurrence, so the
+// compiler keeps several tokens' operands in flight
+template <typename T>
+__global__ void rglru_scan_kernel(const float* __restrict__ gates, const float* __restrict__ u, const T* __restrict__ ypre,
+                                  int64_t y_stride, const T* __restrict__ lam, float cmul, int channels, int blocks,
+                                  const int32_t* __restrict__ cu_q, const int32_t* __restrict__ ctx0,
+                                  const int32_t* __restrict__ slot, int64_t n, float* __restrict__ S, T* __restrict__ out) {
+  const int s = blockIdx.y;
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= channels) return;
+  const int64_t q0 = cu_q[s], q1 = cu_q[s + 1];
+  if (q1 <= q0) return;
+  const int bw = channels / blocks, blk = c / bw, cc = c - blk * bw;
+  const float sp = softplusf_(ldf(lam + c));
+  float* sp_state = S + (int64_t)slot[s] * channels + c;
+  float st = ctx0[s] == 0 ? 0.f : *sp_state;
+  const float* gp = gates + ((int64_t)blk * n) * (2 * bw) + cc;
+#pragma unroll 4
+  for (int64_t t = q0; t < q1; ++t) {
+    const float gr = gp[t * (2 * bw)], gi = gp[t * (2 * bw) + bw];
+    const float uv = u[t * channels + c];
+    const float yv = gelu_tanhf_(ldf(ypre + t * y_stride + c));
+    const float r = 1.f / (1.f + expf(-gr)), ig = 1.f / (1.f + expf(-gi));
+    const float log_a = -cmul * r * sp;
+    const float a = expf(log_a);
+    const float mult = sqrtf(fmaxf(-expm1f(2.f * log_a), 0.f));     // sqrt(1 - a^2), without cancellation near a = 1
+    st = a * st + mult * (ig * uv);
+    stf(out + t * channels + c, st * yv);
+  }
+  *sp_state = st;
+}
+
+// ---- state-space-duality recurrence -------------------------------------------------------------------------------
+// one workgroup per (portion, head): blockDim = (P, NG); thread (p, g) keeps S[n, p] for n = g, g + NG, ... in registers.
+// Per token: S <- dA S + dt B[n] x[p]; partial y[p] = sum over own n of S C[n]; partials meet in LDS.
+constexpr int SSD_R = 16;      // state entries per thread
+constexpr int SSD_TB = 4;      // tokens per LDS round
+
+template <typename T>
+__global__ void ssd_scan_kernel(const float* __restrict__ xbc, const T* __restrict__ proj, int64_t proj_stride, int64_t dt_col,
+                                const T* __restrict__ dt_bias, const T* __restrict__ A_log, const T* __restrict__ Dp, int heads,
+                                int P, int N, int G, const int32_t* __restrict__ cu_q, const int32_t* __restrict__ ctx0,
+                                const int32_t* __restrict__ slot, float* __restrict__ S, float* __restrict__ y) {
+  extern __shared__ float part[];                   // [SSD_TB][NG][P]
+  const int s = blockIdx.y, h = blockIdx.x;
+  const int p = threadIdx.x, g = threadIdx.y, NG = blockDim.y;
+  const int64_t q0 = cu_q[s], q1 = cu_q[s + 1];
+  if (q1 <= q0) return;
+  const int inner = heads * P, grp = h / (heads / G);
+  const int64_t row = inner + 2 * G * N;
+  const float A = -expf(ldf(A_log + h)), Dh = ldf(Dp + h), dtb = ldf(dt_bias + h);
+  float* Sh = S + (((int64_t)slot[s] * heads + h) * N) * P;
+  float st[SSD_R];
+  const bool fresh = ctx0[s] == 0;
+#pragma unroll
+  for (int r = 0; r < SSD_R; ++r) {
+    const int nn = g + r * NG;
+    st[r] = (!fresh && nn < N) ? Sh[(int64_t)nn * P + p] : 0.f;
+  }
+  for (int64_t tb = q0; tb < q1; tb += SSD_TB) {
+    const int cnt = (int)((q1 - tb) < SSD_TB ? (q1 - tb) : SSD_TB);
+    for (int k = 0; k < cnt; ++k) {
+      const int64_t t = tb + k;
+      const float* rowp = xbc + t * row;
+      const float dt = softplusf_(ldf(proj + t * proj_stride + dt_col + h) + dtb);
+      const float dA = expf(A * dt);
+      const float xv = rowp[h * P + p];
+      const float* Bp = rowp + inner + grp * N;
+      const float* Cp = rowp + inner + G * N + grp * N;
+      float acc = 0.f;
+#pragma unroll
+      for (int r = 0; r < SSD_R; ++r) {
+        const int nn = g + r * NG;
+        if (nn < N) {
+          st[r] = dA * st[r] + (dt * Bp[nn]) * xv;
+          acc += st[r] * Cp[nn];
+        }
+      }
+      part[(k * NG + g) * P + p] = acc;
+    }
+    __syncthreads();
+    // thread (p, g) finishes token g of the round (NG >= SSD_TB is guaranteed by the launcher, or loops)
+    for (int k = g; k < cnt; k += NG) {
+      float acc = 0.f;
+      for (int gg = 0; gg < NG; ++gg) acc += part[(k * NG + gg) * P + p];
+      const int64_t t = tb + k;
+      y[t * inner + h * P + p] = acc + Dh * xbc[t * row + h * P + p];
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int r = 0; r < SSD_R; ++r) {
+    const int nn = g + r * NG;
+    if (nn < N) Sh[(int64_t)nn * P + p] = st[r];
+  }
+}
+
+// ---- gate, then group RMS norm ------------------------------------------------------------------------------------
+// one workgroup per (token, group)
+template <typename T>
+__global__ void gated_group_norm_kernel(const float* __restrict__ y, const T* __restrict__ z, int64_t z_stride,
+                                        const T* __restrict__ w, int inner, int groups, float eps, T* __restrict__ out) {
+  __shared__ float red[16];
+  const int64_t t = blockIdx.y;
+  const int gsz = inner / groups, c0 = blockIdx.x * gsz;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < gsz; c += blockDim.x) {
+    const float v = y[t * inner + c0 + c] * siluf_(ldf(z + t * z_stride + c0 + c));
+    ss += v * v;
+  }
+  const float r = rsqrtf(block_sum(ss, red) / (float)gsz + eps);
+  for (int c = threadIdx.x; c < gsz; c += blockDim.x) {
+    const float v = y[t * inner + c0 + c] * siluf_(ldf(z + t * z_stride + c0 + c));
+    stf(out + t * inner + c0 + c, v * r * ldf(w + c0 + c));
+  }
+}
+
+}  // namespace
+
+extern "C" int nvs_causal_conv(const void* in, int64_t in_stride, int dtype, const void* w, const void* b, int channels, int taps,
+                               int act, const int32_t* cu_q, const int32_t* ctx0, const int32_t* slot, const int32_t* tseq, int nseq,
+                               int64_t n, float* state, float* out, void* stream) {
+  NVS_REQUIRE(in && w && cu_q && ctx0 && slot && tseq && state && out, "nvs_causal_conv: null argument");
+  NVS_REQUIRE(channels > 0 && taps >= 1 && taps <= MAX_TAPS && in_stride >= channels && nseq >= 0 && n >= 0 && (act == 0 || act == 1),
+              "nvs_causal_conv: channels %d taps %d (1..%d) stride %lld act %d", channels, taps, MAX_TAPS, (long long)in_stride, act);
+  if (n == 0 || nseq == 0) return NVS_OK;
+  NVS_REQUIRE(n <= 65535 * 64ll && nseq <= 65535, "nvs_causal_conv: step too large");
+  const dim3 block(channels >= 256 ? 256 : 64);
+  const unsigned gx = (channels + block.x - 1) / block.x;
+  // grid.y is limited to 65535: larger steps go in slices
+  for (int64_t t0 = 0; t0 < n; t0 += 65535) {
+    const int64_t cnt = n - t0 < 65535 ? n - t0 : 65535;
+    NVS_DISPATCH(dtype, causal_conv_kernel<T><<<dim3(gx, (unsigned)cnt), block, 0, (hipStream_t)stream>>>(
+                            (const T*)in, in_stride, (const T*)w, (const T*)b, channels, taps, act, cu_q, ctx0, slot, tseq, state, out,
+                            t0));
+  }
+  int rc = nvs_check_launch("nvs_causal_conv");
+  if (rc) return rc;
+  if (taps > 1) {
+    NVS_DISPATCH(dtype, conv_state_kernel<T><<<dim3(gx, (unsigned)nseq), block, 0, (hipStream_t)stream>>>(
+                            (const T*)in, in_stride, channels, taps, cu_q, ctx0, slot, state));
+    rc = nvs_check_launch("nvs_causal_conv (state)");
+  }
+  return rc;
+}
+
+extern "C" int nvs_rglru_scan(const float* gates, const float* u, const void* ypre, int64_t y_stride, int dtype, const void* lam,
+                              float c, int channels, int blocks, const int32_t* cu_q, const int32_t* ctx0, const int32_t* slot, int nseq,
+                              int64_t n, float* S, void* out, void* stream) {
+  NVS_REQUIRE(gates && u && ypre && lam && cu_q && ctx0 && slot && S && out, "nvs_rglru_scan: null argument");
+  NVS_REQUIRE(channels > 0 && blocks > 0 && channels % blocks == 0 && y_stride >= channels && nseq >= 0 && nseq <= 65535 && n >= 0,
+              "nvs_rglru_scan: channels %d blocks %d", channels, blocks);
+  if (n == 0 || nseq == 0) return NVS_OK;
+  const dim3 block(64);
+  NVS_DISPATCH(dtype, rglru_scan_kernel<T><<<dim3((channels + 63) / 64, (unsigned)nseq), block, 0, (hipStream_t)stream>>>(
+                          gates, u, (const T*)ypre, y_stride, (const T*)lam, c, channels, blocks, cu_q, ctx0, slot, n, S, (T*)out));
+  return nvs_check_launch("nvs_rglru_scan");
+}
+
+extern "C" int nvs_ssd_scan(const float* xbc, const void* proj, int64_t proj_stride, int64_t dt_col, int dtype, const void* dt_bias,
+                            const void* A_log, const void* D, int heads, int P, int N, int G, const int32_t* cu_q, const int32_t* ctx0,
+                            const int32_t* slot, int nseq, int64_t n, float* S, float* y, void* stream) {
+  NVS_REQUIRE(xbc && proj && dt_bias && A_log && D && cu_q && ctx0 && slot && S && y, "nvs_ssd_scan: null argument");
+  NVS_REQUIRE(heads > 0 && G > 0 && heads % G == 0 && P > 0 && P <= 256 && N > 0 && nseq >= 0 && nseq <= 65535,
+              "nvs_ssd_scan: heads %d groups %d head size %d state %d", heads, G, P, N);
+  if (n == 0 || nseq == 0) return NVS_OK;
+  int ng = 1024 / P;
+  if (ng > N) ng = N;
+  NVS_REQUIRE(ng * SSD_R >= N, "nvs_ssd_scan: state %d x head size %d exceeds one workgroup's registers", N, P);
+  // no more rows of threads than needed to hold the state, but at least enough to spread the per-round reduction
+  int need = (N + SSD_R - 1) / SSD_R;
+  if (need < SSD_TB) need = SSD_TB < ng ? SSD_TB : ng;
+  ng = need;
+  const size_t lds = (size_t)SSD_TB * ng * P * sizeof(float);
+  NVS_DISPATCH(dtype, ssd_scan_kernel<T><<<dim3(heads, (unsigned)nseq), dim3(P, ng), lds, (hipStream_t)stream>>>(
+                          xbc, (const T*)proj, proj_stride, dt_col, (const T*)dt_bias, (const T*)A_log, (const T*)D, heads, P, N, G, cu_q,
+                          ctx0, slot, S, y));
+  return nvs_check_launch("nvs_ssd_scan");
+}
+
+extern "C" int nvs_gated_group_norm(const float* y, const void* z, int64_t z_stride, int dtype, const void* w, int inner, int groups,
+                                    float eps, int64_t n, void* out, void* stream) {
+  NVS_REQUIRE(y && z && w && out && inner > 0 && groups > 0 && inner % groups == 0 && z_stride >= inner && n >= 0,
+              "nvs_gated_group_norm: inner %d groups %d", inner, groups);
+  if (n == 0) return NVS_OK;
+  NVS_REQUIRE(n <= 65535ll * 65535ll, "nvs_gated_group_norm: step too large");
+  const int gsz = inner / groups;
+  const dim3 block(gsz >= 1024 ? 256 : (gsz >= 128 ? 128 : 64));
+  for (int64_t t0 = 0; t0 < n; t0 += 65535) {
+    const int64_t cnt = n - t0 < 65535 ? n - t0 : 65535;
+    NVS_DISPATCH(dtype, gated_group_norm_kernel<T><<<dim3(groups, (unsigned)cnt), block, 0, (hipStream_t)stream>>>(
+                            y + t0 * inner, (const T*)z + t0 * z_stride, z_stride, (const T*)w, inner, groups, eps, (T*)out + t0 * inner));
+  }
+  return nvs_check_launch("nvs_gated_group_norm");
+}

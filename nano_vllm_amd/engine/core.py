@@ -61,18 +61,33 @@ class LLMEngine:
                 self.ps.append(proc)
         from .runner import ModelRunner
         self.model_runner = ModelRunner(config, 0)                  # also fills config.num_kvcache_blocks
-        from transformers import AutoTokenizer
-        self.tokenizer = AutoTokenizer.from_pretrained(config.model, use_fast=True)
-        config.eos = self.tokenizer.eos_token_id if self.tokenizer.eos_token_id is not None else -1
+        self.tokenizer = self._load_tokenizer(config)
+        if self.tokenizer is not None:
+            config.eos = self.tokenizer.eos_token_id if self.tokenizer.eos_token_id is not None else -1
+        else:
+            eos = getattr(config.hf_config, "eos_token_id", -1)
+            config.eos = eos if isinstance(eos, int) else -1
         self.scheduler = Scheduler(config)
         # decode lookahead (see _step_lookahead), at any TP degree: workers execute the staging images rank 0
         # posts, and every rank holds the sampled ids on the device. NVL_LOOKAHEAD=0 restores the strictly
         # serial loop for A/B measurements
-        self._lookahead = os.environ.get("NVL_LOOKAHEAD", "1") != "0"
+        # (stateful families run every step through the packed varlen path, which has no split begin / end form)
+        self._lookahead = os.environ.get("NVL_LOOKAHEAD", "1") != "0" and not self.scheduler.stateful
+        self._replay: dict = {}            # request name -> Sequence of a caller-fixed schedule (replay_step)
         self._unfilled = None              # sequences of an in-flight lookahead step whose token values are pending
         self._requests = 0                 # ordinal of the next request (the sampler's per-sequence key)
         self._exited = False
         atexit.register(self.exit)
+
+    @staticmethod
+    def _load_tokenizer(config):
+        """The checkpoint's tokenizer, or None for a directory that ships none (requests are token ids then, and results
+        carry an empty "text")."""
+        names = ("tokenizer.json", "tokenizer_config.json", "vocab.json", "tokenizer.model")
+        if not any(os.path.exists(os.path.join(config.model, n)) for n in names):
+            return None
+        from transformers import AutoTokenizer
+        return AutoTokenizer.from_pretrained(config.model, use_fast=True)
 
     @classmethod
     def worker(cls, model, **kwargs) -> None:
@@ -99,6 +114,7 @@ class LLMEngine:
     def _checked_prompt(self, prompt: str | list[int], sampling_params: SamplingParams) -> list[int]:
         """Tokenise and validate one request; no side effects."""
         if isinstance(prompt, str):
+            assert self.tokenizer is not None, "this checkpoint ships no tokenizer: pass token ids"
             prompt = self.tokenizer.encode(prompt)
         assert len(prompt) > 0, "empty prompt"
         # the staging block tables and the RoPE table are sized by max_model_len: a request that would outgrow
@@ -223,7 +239,43 @@ class LLMEngine:
                 pbar.update(1)
         pbar.close()
         ordered = [done[k] for k in sorted(done)]
-        return [{"text": self.tokenizer.decode(toks), "token_ids": toks} for toks in ordered]
+        decode = self.tokenizer.decode if self.tokenizer is not None else (lambda toks: "")
+        return [{"text": decode(toks), "token_ids": toks} for toks in ordered]
+
+    # ------------------------------------------------------------------ a schedule fixed by the caller
+    def replay_step(self, entries: list[dict], end: list = ()):
+        """Run ONE engine step whose contents the caller fixes, and return logits instead of sampling: the way to replay a
+        recorded schedule, or to drive the engine from an external scheduler. `entries`: dicts with "id" (any hashable
+        request name), "tokens" (the request's NEXT token ids) and optionally "want" (indices into these tokens whose
+        logits are returned; default none). All entries form one batch — portions of prompts beside single tokens. A request
+        is admitted at its first entry and may sit out steps; `end` names the requests that are over after this step (their
+        pages and state slots return to the pools). Pages, state slots and the step itself are the scheduler's, the block
+        manager's and the runner's, as in generate(). Returns float32 logits [total wanted, vocab] (host), in entry order.
+        Stateful families only (the paged-KV transformer path samples inside its captured step)."""
+        assert self.scheduler.stateful, "replay_step drives the packed varlen step path of stateful model families"
+        portions, want = [], []
+        for e in entries:
+            toks = [int(t) for t in e["tokens"]]
+            assert toks, "an entry brings at least one token"
+            seq = self._replay.get(e["id"])
+            if seq is None:
+                seq = self._replay[e["id"]] = self._new_sequence(toks, SamplingParams(temperature=0.0, max_tokens=1))
+            else:
+                assert seq.num_cached_tokens == seq.num_tokens
+                for t in toks:
+                    seq.append_token(t)
+            assert seq.num_tokens <= self.config.max_model_len, "request outgrows max_model_len"
+            portions.append((seq, len(toks)))
+            want.append([int(w) for w in e.get("want", ())])
+        assert sum(c for _, c in portions) <= self.config.max_num_batched_tokens, "step exceeds max_num_batched_tokens"
+        batch = self.scheduler.schedule_portions(portions)
+        logits = self.model_runner.call("run_logits", batch, want)
+        self.scheduler.finish_portions(batch)
+        for name in end:
+            seq = self._replay.pop(name, None)
+            if seq is not None:
+                self.scheduler.retire(seq)
+        return logits
 
 
 class LLM(LLMEngine):

@@ -24,10 +24,13 @@ _NIL = -1
 
 class BlockManager:
 
-    def __init__(self, num_blocks: int, block_size: int):
+    def __init__(self, num_blocks: int, block_size: int, prefix_cache: bool = True):
+        """`prefix_cache=False` (stateful models: a prefix's pages are useless without the state that went with them):
+        no block is ever hashed, found or revived; allocation order and everything else is unchanged."""
         assert num_blocks > 0
         self.num_blocks = num_blocks
         self.block_size = block_size
+        self.prefix_cache = prefix_cache
         self.ref_count = [0] * num_blocks
         self.block_hash = [-1] * num_blocks
         self.block_tokens: list[bytes | None] = [None] * num_blocks   # int64 bytes of the hashed tokens
@@ -106,6 +109,8 @@ class BlockManager:
     def _probe_prefix(self, seq: Sequence):
         """Walk the hash chain over all blocks but the last (block_manager.py:62-70)."""
         hashes, ids = [], []
+        if not self.prefix_cache:
+            return hashes, ids
         h = -1
         bs = self.block_size
         toks = seq.token_ids
@@ -168,8 +173,27 @@ class BlockManager:
         if seq.num_tokens % self.block_size == 1:
             seq.block_table.append(self._allocate_block())
 
+    # --- growth by portions: a sequence whose tokens arrive step by step (a caller-fixed schedule) -------------------
+    def blocks_to_extend(self, seq: Sequence, num_tokens: int) -> int:
+        """Blocks missing for the sequence to hold `num_tokens` tokens."""
+        return max(0, -(-num_tokens // self.block_size) - len(seq.block_table))
+
+    def can_extend(self, seq: Sequence, num_tokens: int) -> bool:
+        return self.num_free >= self.blocks_to_extend(seq, num_tokens)
+
+    def extend(self, seq: Sequence, num_tokens: int) -> None:
+        """Append blocks until the table covers `num_tokens` tokens (no prefix lookup: the sequence is already running)."""
+        fresh = not seq.block_table
+        for _ in range(self.blocks_to_extend(seq, num_tokens)):
+            seq.block_table.append(self._allocate_block())
+        if fresh:
+            self._table_gen += 1
+            seq.table_gen = self._table_gen
+
     def hash_blocks(self, seq: Sequence) -> None:
         """Register every block that became full in this step (:110-120)."""
+        if not self.prefix_cache:
+            return
         bs = self.block_size
         start = seq.num_cached_tokens // bs
         end = (seq.num_cached_tokens + seq.num_scheduled_tokens) // bs

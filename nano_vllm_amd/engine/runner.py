@@ -37,7 +37,7 @@ from .. import ops
 from ..api import Config, model_geometry
 from ..attn_meta import get_context, reset_context, set_context
 from ..layers import Sampler
-from ..qwen3 import Qwen3ForCausalLM
+from ..registry import spec_of
 from ..weights import init_dummy_weights, load_model
 from .seq import Sequence
 
@@ -263,7 +263,9 @@ class ModelRunner:
         self.world_size = config.tensor_parallel_size
         self.rank = rank
         assert torch.cuda.is_available(), "nano_vllm_amd needs a HIP device (no CPU fallback for the hot path)"
-        ops.load_library()
+        self.spec = spec_of(hf)                 # model family: class, cache layout, step path (registry.py)
+        if not self.spec.stateful:
+            ops.load_library()                  # (stateful families run on libnvl_seq.so; the sampler loads this one on first use)
 
         # Devices: rank r drives GPU r, as the reference does (model_runner.py:27). NVL_TP_SHARE_GPU=1 puts every
         # rank on GPU 0 — the functional test of the TP engine on a one-GPU box (with NVL_TP_BACKEND=gloo:
@@ -297,6 +299,8 @@ class ModelRunner:
     def _init_rest(self, config: Config, hf, rank: int):
         from .. import tp
         tp.init(rank if self.world_size > 1 else 0, self.world_size)
+        if self.spec.stateful:
+            return self._init_stateful(config, hf)
         self.geo = model_geometry(hf, self.world_size)
         dtype = self.geo["dtype"] or torch.bfloat16
         if isinstance(dtype, str):
@@ -312,7 +316,7 @@ class ModelRunner:
         torch.set_default_dtype(dtype)
         torch.set_default_device(self.device)
         try:
-            self.model = Qwen3ForCausalLM(hf)
+            self.model = self.spec.build(hf)
             if config.dummy_weights:
                 init_dummy_weights(self.model, hf, config.seed)
             else:
@@ -828,7 +832,151 @@ class ModelRunner:
         return self.tokens_host[:ns].tolist()
 
     def run(self, seqs: list[Sequence], is_prefill: bool) -> list[int] | None:
+        if self.spec.stateful:
+            return self.run_portions(seqs)
         return self._run_prefill(seqs) if is_prefill else self._run_decode(seqs)
+
+    # ------------------------------------------------------------------ stateful families: one packed varlen step path
+    def _init_stateful(self, config: Config, hf):
+        """Models whose layers carry per-sequence state (registry.ModelSpec.stateful). What differs from the paged-KV
+        transformer path: pages exist only for the layers that attend, with that layer's own head sizes ([pages * block, G, d]
+        keys, [.., G, dv] values, token-major); every stateful layer gets `[max_num_seqs, ...]` 32-bit state tensors indexed
+        by the sequence's state slot; and there is ONE step path — every scheduled sequence contributes its next
+        `num_scheduled_tokens` tokens (a portion of a prompt or one decoded token) to a packed batch, so prefill, chunked
+        prefill, decode and any mix of them are the same launches. Steps run eagerly."""
+        dtype = getattr(torch, "bfloat16" if config.dtype == "auto" else config.dtype)
+        self.dtype = dtype
+        self.p2p = False
+        self.chan = None
+        self.graphs, self.graphs_px = {}, {}
+        hf.kvcache_block_size = self.block_size
+        prev_dtype = torch.get_default_dtype()
+        torch.set_default_dtype(dtype)
+        torch.set_default_device(self.device)
+        try:
+            with torch.inference_mode():
+                self.model = self.spec.build(hf, dtype)
+                if config.dummy_weights:
+                    self.model.init_random(config.seed)
+                else:
+                    load_model(self.model, config.model)
+            self.geo = self.model.geo
+            self.sampler = None                                   # made on the first sampled step
+            cfg = self.config
+            self.max_bs = cfg.max_num_seqs
+            self.max_blocks = -(-cfg.max_model_len // self.block_size)
+            nt, ns, w = cfg.max_num_batched_tokens, min(cfg.max_num_seqs, cfg.max_num_batched_tokens), self.max_blocks
+            self.sstage = _Stage([
+                ("ids", np.int64, (nt,)), ("pos", np.int64, (nt,)), ("rng", np.uint64, (2,)), ("rkey", np.int64, (ns,)),
+                ("slots", np.int32, (nt,)), ("tseq", np.int32, (nt,)), ("rows", np.int32, (nt,)), ("cu_q", np.int32, (ns + 1,)),
+                ("ctx0", np.int32, (ns,)), ("sslot", np.int32, (ns,)), ("temps", np.float32, (ns,)), ("bt", np.int32, (ns, w)),
+            ], self.device)
+            self.step_count = 0
+            self.tokens_dev = torch.zeros(ns, dtype=torch.int64, device=self.device)
+            self.tokens_host = torch.zeros(ns, dtype=torch.int64, device="cpu", pin_memory=True)
+            self._allocate_stateful_caches()
+        finally:
+            torch.set_default_device("cpu")
+            torch.set_default_dtype(prev_dtype)
+
+    def _allocate_stateful_caches(self):
+        cfg = self.config
+        kv_layers = [m for m in self.model.modules() if hasattr(m, "kv_shapes")]
+        st_layers = [m for m in self.model.modules() if hasattr(m, "state_shapes")]
+        esize = torch.finfo(self.dtype).bits // 8
+        per_token = sum(int(np.prod(k)) + int(np.prod(v)) for k, v in (m.kv_shapes() for m in kv_layers)) * esize
+        block_bytes = max(per_token * self.block_size, 1)
+        for m in st_layers:                                       # state first: small, and it is not optional
+            for name, shape in m.state_shapes().items():
+                setattr(m, name, torch.zeros(cfg.max_num_seqs, *shape, dtype=torch.float32, device=self.device))
+        if cfg.num_kvcache_blocks <= 0:
+            free, total = torch.cuda.mem_get_info()
+            # no profiling pass (it would need pages): activations of the largest step are bounded by the widest fused
+            # projection, held a few times over in 32-bit
+            widest = max([p.shape[0] for p in self.model.parameters() if p.dim() == 2] + [1])
+            reserve = cfg.max_num_batched_tokens * widest * 16 + (1 << 30)
+            budget = free - (total * (1.0 - cfg.gpu_memory_utilization)) - reserve
+            need_all = cfg.max_num_seqs * (-(-cfg.max_model_len // self.block_size))   # more pages than this are never used
+            cfg.num_kvcache_blocks = int(min(budget // block_bytes, need_all))
+        assert cfg.num_kvcache_blocks > 0, "no memory left for the KV cache"
+        slots = cfg.num_kvcache_blocks * self.block_size
+        for m in kv_layers:
+            ks, vs = m.kv_shapes()
+            m.k_cache = torch.zeros(slots, *ks, dtype=self.dtype, device=self.device)
+            m.v_cache = torch.zeros(slots, *vs, dtype=self.dtype, device=self.device)
+            m.block_size = self.block_size
+
+    def prepare_portions(self, seqs: list[Sequence], want: list[list[int]] | None = None) -> dict:
+        """Fill the staging block for a packed step: sequence i contributes tokens [num_cached_tokens, + num_scheduled_tokens).
+        `want[i]`: indices INSIDE portion i whose logits the caller asks for (default: the portion's last token)."""
+        st = self.sstage
+        ev = st.uploaded[0]
+        if ev is not None:
+            ev.synchronize()
+        a, bs = st.np, self.block_size
+        n = nrows = 0
+        a["cu_q"][0] = 0
+        for i, seq in enumerate(seqs):
+            start, lq = seq.num_cached_tokens, seq.num_scheduled_tokens
+            end = start + lq
+            assert lq >= 1 and seq.state_slot >= 0 and len(seq.block_table) * bs >= end
+            a["ids"][n:n + lq] = seq.token_ids[start:end]
+            pos = np.arange(start, end, dtype=np.int64)
+            a["pos"][n:n + lq] = pos
+            table = np.asarray(seq.block_table, dtype=np.int64)
+            a["slots"][n:n + lq] = table[pos // bs] * bs + pos % bs
+            a["tseq"][n:n + lq] = i
+            a["cu_q"][i + 1] = n + lq
+            a["ctx0"][i] = start
+            a["sslot"][i] = seq.state_slot
+            a["temps"][i] = seq.temperature
+            a["rkey"][i] = seq.rng_key | (end << 32)
+            a["bt"][i, :len(table)] = table
+            a["bt"][i, len(table):] = -1
+            rows = [lq - 1] if want is None else want[i]
+            for r in rows:
+                assert 0 <= r < lq
+                a["rows"][nrows] = n + r
+                nrows += 1
+            n += lq
+        return dict(n=n, ns=len(seqs), nrows=nrows)
+
+    @torch.inference_mode()
+    def _launch_portions(self, info: dict) -> torch.Tensor:
+        """Upload the staged step and run the model; returns the logits of the staged rows (on the device)."""
+        from ..ops_seq import Portions
+        st = self.sstage
+        st.upload()
+        t = st.t
+        n, ns, nrows = info["n"], info["ns"], info["nrows"]
+        por = Portions(t["cu_q"], t["ctx0"], t["sslot"], t["tseq"], ns, n)
+        set_context(True, slot_mapping=t["slots"][:n], block_tables=t["bt"][:ns], portions=por)
+        x = self.model(t["ids"][:n], t["pos"][:n])
+        logits = self.model.compute_logits(x, t["rows"], nrows)
+        reset_context()
+        return logits
+
+    def run_portions(self, seqs: list[Sequence]) -> list[int]:
+        """One packed step, one sampled token per sequence (from its portion's last token)."""
+        info = self.prepare_portions(seqs)
+        self._next_rng(self.sstage)
+        logits = self._launch_portions(info)
+        ns, t = info["ns"], self.sstage.t
+        if self.sampler is None:
+            ops.load_library()
+            self.sampler = Sampler(seed=self.config.seed, max_rows=self.config.max_num_seqs)
+        with torch.inference_mode():
+            self.sampler(logits, t["temps"][:ns], out=self.tokens_dev[:ns], offset_dev=t["rng"][:1], row_keys=t["rkey"][:ns])
+        self.tokens_host[:ns].copy_(self.tokens_dev[:ns], non_blocking=True)
+        torch.cuda.current_stream().synchronize()
+        return self.tokens_host[:ns].tolist()
+
+    def run_logits(self, seqs: list[Sequence], want: list[list[int]]) -> np.ndarray:
+        """One packed step without sampling: float32 logits [rows wanted, vocab] on the host, in the order of `seqs` and `want`."""
+        info = self.prepare_portions(seqs, want)
+        logits = self._launch_portions(info)
+        out = logits.float().cpu().numpy()
+        return out
 
     # ------------------------------------------------------------------ hipGraph capture
     @torch.inference_mode()

@@ -26,7 +26,16 @@ class Scheduler:
         self.max_num_batched_tokens = config.max_num_batched_tokens
         self.eos = config.eos
         self.block_size = config.kvcache_block_size
-        self.block_manager = BlockManager(config.num_kvcache_blocks, config.kvcache_block_size)
+        # stateful models (registry.ModelSpec.stateful): no prefix cache, and every sequence holds a state slot while it
+        # holds pages — the runner has max_num_seqs of them, so a slot is always free when a sequence can be admitted
+        from ..registry import spec_of
+        hf = getattr(config, "hf_config", None)
+        self.stateful = spec_of(hf).stateful if hf is not None else False
+        self.block_manager = BlockManager(config.num_kvcache_blocks, config.kvcache_block_size, prefix_cache=not self.stateful)
+        self.state_slots = None
+        if self.stateful:
+            from .state_slots import StateSlotManager
+            self.state_slots = StateSlotManager(config.max_num_seqs)
         self.waiting: deque[Sequence] = deque()
         self.running: deque[Sequence] = deque()
 
@@ -53,8 +62,8 @@ class Scheduler:
             fresh = not seq.block_table
             if fresh:
                 cached_blocks = bm.can_allocate(seq)
-                if cached_blocks < 0:
-                    break                                    # pool exhausted: head-of-line blocks
+                if cached_blocks < 0 or (self.state_slots is not None and not self.state_slots.can_allocate()):
+                    break                                    # pool (or state slots) exhausted: head-of-line blocks
                 todo = seq.num_tokens - cached_blocks * bs
             else:                                            # continuation of a chunked prefill
                 todo = seq.num_tokens - seq.num_cached_tokens
@@ -62,6 +71,8 @@ class Scheduler:
                 break                                        # only the first sequence may be chunked
             if fresh:
                 bm.allocate(seq, cached_blocks)              # blocks for the WHOLE sequence
+                if self.state_slots is not None:
+                    self.state_slots.allocate(seq)
             seq.num_scheduled_tokens = min(todo, budget)
             budget -= seq.num_scheduled_tokens
             if seq.num_cached_tokens + seq.num_scheduled_tokens == seq.num_tokens:
@@ -97,8 +108,52 @@ class Scheduler:
     def preempt(self, seq: Sequence) -> None:
         seq.status = SequenceStatus.WAITING
         seq.is_prefill = True
-        self.block_manager.deallocate(seq)
+        self._release(seq)
         self.waiting.appendleft(seq)
+
+    def _release(self, seq: Sequence) -> None:
+        """Give back what a sequence holds: its pages and, for stateful models, its state slot."""
+        self.block_manager.deallocate(seq)
+        if self.state_slots is not None:
+            self.state_slots.release(seq)
+
+    # --- a step whose contents the caller fixes (replaying a recorded schedule, an external scheduler) --------------------
+    def schedule_portions(self, portions: list[tuple[Sequence, int]]) -> list[Sequence]:
+        """One step made of the given (sequence, number of its next tokens) pairs, in that order: portions of prompts and
+        single decoded tokens side by side. A sequence is admitted at its first portion (pages for the tokens it has so far,
+        a state slot for stateful models) and its table grows as its tokens arrive. Raises if the pool cannot hold the step:
+        a caller that fixes the schedule has also fixed what must fit."""
+        bm = self.block_manager
+        batch = []
+        for seq, count in portions:
+            assert count >= 1 and seq.num_cached_tokens + count <= seq.num_tokens
+            end = seq.num_cached_tokens + count
+            if not bm.can_extend(seq, end):
+                raise RuntimeError(f"KV pool exhausted: sequence {seq.seq_id} needs {bm.blocks_to_extend(seq, end)} more blocks, "
+                                   f"{bm.num_free} free")
+            if seq.state_slot < 0 and self.state_slots is not None:
+                if not self.state_slots.can_allocate():
+                    raise RuntimeError("no free state slot: more live sequences than max_num_seqs")
+                self.state_slots.allocate(seq)
+            bm.extend(seq, end)
+            if seq.status is SequenceStatus.WAITING:
+                seq.status = SequenceStatus.RUNNING
+                self.running.append(seq)
+            seq.num_scheduled_tokens = count
+            batch.append(seq)
+        return batch
+
+    def finish_portions(self, batch: list[Sequence]) -> None:
+        """Account a caller-fixed step as done (no token is appended: the caller owns the tokens)."""
+        for seq in batch:
+            seq.num_cached_tokens += seq.num_scheduled_tokens
+            seq.num_scheduled_tokens = 0
+
+    def retire(self, seq: Sequence) -> None:
+        """End a sequence of a caller-fixed schedule: its pages and state slot go back to the pools."""
+        seq.status = SequenceStatus.FINISHED
+        self._release(seq)
+        self.running = deque(s for s in self.running if s is not seq)
 
     # --- lookahead form of postprocess for decode steps: `postprocess_early` does everything `postprocess` does that
     # cannot depend on the sampled values — hash -> count -> append a PLACEHOLDER -> finish by max_tokens / deallocate —
@@ -129,7 +184,7 @@ class Scheduler:
             if not seq.ignore_eos and token_id == self.eos and seq.status is not SequenceStatus.FINISHED:
                 seq.status = SequenceStatus.FINISHED
                 if seq.block_table:               # (a preempted sequence holds no blocks)
-                    self.block_manager.deallocate(seq)
+                    self._release(seq)
                 finished = True
         if finished:
             self.running = deque(s for s in self.running if s.status is not SequenceStatus.FINISHED)
@@ -148,7 +203,7 @@ class Scheduler:
             if (check_eos and not seq.ignore_eos and token_id == self.eos) or \
                     seq.num_completion_tokens == seq.max_tokens:
                 seq.status = SequenceStatus.FINISHED
-                bm.deallocate(seq)
+                self._release(seq)
                 finished = True
         if finished:
             self.running = deque(s for s in self.running if s.status is not SequenceStatus.FINISHED)

@@ -24,7 +24,7 @@ class SequenceStatus(Enum):
 class Sequence:
     __slots__ = ("seq_id", "status", "token_ids", "last_token", "num_tokens", "num_prompt_tokens",
                  "num_cached_tokens", "num_scheduled_tokens", "is_prefill", "block_table", "table_gen",
-                 "temperature", "max_tokens", "ignore_eos", "rng_key")
+                 "temperature", "max_tokens", "ignore_eos", "rng_key", "state_slot")
 
     block_size = 256          # set by the engine from Config.kvcache_block_size
     counter = count()
@@ -44,6 +44,7 @@ class Sequence:
         self.num_scheduled_tokens = 0
         self.is_prefill = True
         self.block_table: list[int] = []
+        self.state_slot = -1          # slot of the per-sequence state of stateful models (engine/state_slots.py); -1: none
         self.table_gen = 0            # stamped by BlockManager.allocate: distinguishes re-allocations of the same length
         self.temperature = sp.temperature
         self.max_tokens = sp.max_tokens
@@ -93,7 +94,7 @@ class Sequence:
     def __getstate__(self):
         payload = self.token_ids if self.is_prefill else self.last_token
         return (self.seq_id, self.num_tokens, self.num_prompt_tokens, self.num_cached_tokens,
-                self.num_scheduled_tokens, self.block_table, self.table_gen, payload)
+                self.num_scheduled_tokens, self.block_table, self.table_gen, payload)      # (state slots: single-process models only)
 
     def __setstate__(self, state):
         (self.seq_id, self.num_tokens, self.num_prompt_tokens, self.num_cached_tokens, self.num_scheduled_tokens,
@@ -105,3 +106,4 @@ class Sequence:
         # fields the workers never read
         self.status, self.is_prefill = SequenceStatus.RUNNING, isinstance(payload, list)
         self.temperature, self.max_tokens, self.ignore_eos = 1.0, 0, False
+        self.state_slot = -1

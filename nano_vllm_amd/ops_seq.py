@@ -1,0 +1,216 @@
+"""ctypes binding of libnvl_seq.so (C ABI in include/nvl_seq.h): the kernels of layers that carry per-sequence state,
+of windowed paged attention with any head size and of norms on a 32-bit residual stream.
+
+As in ops.py, PyTorch owns memory and the stream and every function hands raw device pointers to a hand-written gfx950
+kernel; there is no fallback. Activation / weight tensors are bfloat16 or float32 (`_code`), state and the residual
+stream are float32. The library is built on first use when it is missing (a fresh checkout), by hipcc, in-tree.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import c_char_p, c_float, c_int, c_int64, c_void_p
+
+import torch
+
+from . import build as _build
+
+ABI_VERSION = 1
+_P, _I, _L, _F = c_void_p, c_int, c_int64, c_float
+
+SIGNATURES = {
+    "nvs_abi_version": (c_int, []),
+    "nvs_last_error": (c_char_p, []),
+    "nvs_embed_sinusoid": (c_int, [_P, _I, _P, _P, _L, _I, _F, _F, _P, _P, _P]),
+    "nvs_norm_residual": (c_int, [_P, _P, _P, _P, _P, _I, _L, _I, _F, _P, _P, _P]),
+    "nvs_scalar_norm_rows": (c_int, [_P, _P, _L, _I, _P, _I, _F, _P, _P]),
+    "nvs_xielu": (c_int, [_P, _P, _F, _I, _L, _P, _P]),
+    "nvs_causal_conv": (c_int, [_P, _L, _I, _P, _P, _I, _I, _I, _P, _P, _P, _P, _I, _L, _P, _P, _P]),
+    "nvs_rglru_scan": (c_int, [_P, _P, _P, _L, _I, _P, _F, _I, _I, _P, _P, _P, _I, _L, _P, _P, _P]),
+    "nvs_ssd_scan": (c_int, [_P, _P, _L, _L, _I, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _I, _L, _P, _P, _P]),
+    "nvs_gated_group_norm": (c_int, [_P, _P, _L, _I, _P, _I, _I, _F, _L, _P, _P]),
+    "nvs_knorm_kvstore": (c_int, [_P, _P, _L, _I, _P, _F, _I, _I, _I, _P, _L, _P, _P, _P]),
+    "nvs_window_attn": (c_int, [_P, _L, _P, _F, _P, _L, _I, _P, _P, _P, _L, _I, _P, _P, _P, _I, _L, _I, _I, _I, _I, _F, _I,
+                                _P, _P]),
+}
+
+_lib = None
+
+
+class NvsError(RuntimeError):
+    pass
+
+
+def load_library() -> ctypes.CDLL:
+    """Load libnvl_seq.so, building it first when the checkout has none (or an older one than its sources)."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    path = _build.build_seq()
+    lib = ctypes.CDLL(path)
+    for name, (restype, argtypes) in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype, fn.argtypes = restype, argtypes
+    if lib.nvs_abi_version() != ABI_VERSION:
+        raise NvsError(f"libnvl_seq.so ABI version {lib.nvs_abi_version()} != binding version {ABI_VERSION}; rebuild")
+    _lib = lib
+    return lib
+
+
+def _check(rc: int) -> None:
+    if rc != 0:
+        raise NvsError(f"nvs error {rc}: {_lib.nvs_last_error().decode()}")
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _code(t: torch.Tensor) -> int:
+    if t.dtype == torch.bfloat16:
+        return 0
+    if t.dtype == torch.float32:
+        return 1
+    raise NvsError(f"unsupported activation dtype {t.dtype} (bfloat16 or float32)")
+
+
+def _ptr(t: torch.Tensor | None) -> int | None:
+    if t is None:
+        return None
+    if not t.is_cuda:
+        raise NvsError("device (HIP) tensors only; the hot path has no CPU fallback")
+    return t.data_ptr()
+
+
+def _same(code_of: torch.Tensor, *others: torch.Tensor | None) -> int:
+    for o in others:
+        if o is not None and o.dtype != code_of.dtype:
+            raise NvsError(f"dtype mismatch: {o.dtype} beside {code_of.dtype}")
+    return _code(code_of)
+
+
+class Portions:
+    """Device-side description of a step's packed portions (see include/nvl_seq.h): cu_q [nseq + 1], ctx0 [nseq],
+    slot [nseq], tseq [n], all int32."""
+    __slots__ = ("cu_q", "ctx0", "slot", "tseq", "nseq", "n")
+
+    def __init__(self, cu_q, ctx0, slot, tseq, nseq: int, n: int):
+        self.cu_q, self.ctx0, self.slot, self.tseq, self.nseq, self.n = cu_q, ctx0, slot, tseq, nseq, n
+        for t in (cu_q, ctx0, slot, tseq):
+            assert t.dtype == torch.int32 and t.is_cuda and t.is_contiguous()
+        assert cu_q.numel() >= nseq + 1 and ctx0.numel() >= nseq and slot.numel() >= nseq and tseq.numel() >= n
+
+
+def embed_sinusoid(table, ids, pos, scale: float, base: float, x: torch.Tensor, xh: torch.Tensor | None):
+    lib = load_library()
+    n, width = ids.numel(), table.shape[1]
+    assert x.dtype == torch.float32 and x.shape == (n, width) and x.is_contiguous() and table.is_contiguous()
+    assert ids.dtype == torch.int64 and pos.dtype == torch.int64 and pos.numel() == n
+    assert xh is None or (xh.shape == x.shape and xh.is_contiguous())
+    _check(lib.nvs_embed_sinusoid(_ptr(table), _same(table, xh), _ptr(ids), _ptr(pos), n, width, scale, base, _ptr(x),
+                                  _ptr(xh), _stream()))
+
+
+def norm_residual(x: torch.Tensor, m: torch.Tensor, g: torch.Tensor, eps: float, xh: torch.Tensor | None,
+                  m2: torch.Tensor | None = None, w1: torch.Tensor | None = None, w2: torch.Tensor | None = None):
+    """x += g * rms(m), or with a second branch x += g * rms((rms(m) w1 + rms(m2) w2) / 2)."""
+    lib = load_library()
+    n, width = x.shape
+    assert x.dtype == torch.float32 and x.is_contiguous() and m.shape == x.shape and m.is_contiguous()
+    assert m2 is None or (m2.shape == x.shape and m2.is_contiguous() and w1.numel() == width and w2.numel() == width)
+    assert xh is None or (xh.shape == x.shape and xh.is_contiguous())
+    _check(lib.nvs_norm_residual(_ptr(m), _ptr(m2), _ptr(w1), _ptr(w2), _ptr(g), _same(m, m2, w1, w2, g, xh), n, width, eps,
+                                 _ptr(x), _ptr(xh), _stream()))
+
+
+def scalar_norm_rows(x: torch.Tensor, rows: torch.Tensor | None, nrows: int, g: torch.Tensor, eps: float, out: torch.Tensor):
+    lib = load_library()
+    assert x.dtype == torch.float32 and x.is_contiguous() and out.is_contiguous() and out.shape == (nrows, x.shape[1])
+    assert rows is None or (rows.dtype == torch.int32 and rows.numel() >= nrows)
+    assert rows is not None or nrows <= x.shape[0]
+    _check(lib.nvs_scalar_norm_rows(_ptr(x), _ptr(rows), nrows, x.shape[1], _ptr(g), _same(out, g), eps, _ptr(out), _stream()))
+
+
+def xielu(z: torch.Tensor, pq: torch.Tensor, beta: float = 0.5) -> torch.Tensor:
+    """In place."""
+    lib = load_library()
+    assert z.is_contiguous() and pq.numel() == 2
+    _check(lib.nvs_xielu(_ptr(z), _ptr(pq), beta, _same(z, pq), z.numel(), _ptr(z), _stream()))
+    return z
+
+
+def causal_conv(inp: torch.Tensor, w: torch.Tensor, b: torch.Tensor | None, act: int, por: Portions, state: torch.Tensor,
+                out: torch.Tensor):
+    """inp: [n, channels] view (unit column stride) of a projection output; state [nslots, taps - 1, channels] fp32."""
+    lib = load_library()
+    channels, taps = w.shape
+    assert inp.shape == (por.n, channels) and inp.stride(1) == 1 and w.is_contiguous()
+    assert state.dtype == torch.float32 and state.is_contiguous() and tuple(state.shape[1:]) == (taps - 1, channels)
+    assert out.dtype == torch.float32 and out.is_contiguous() and out.shape == (por.n, channels)
+    _check(lib.nvs_causal_conv(_ptr(inp), inp.stride(0), _same(inp, w, b), _ptr(w), _ptr(b), channels, taps, act, _ptr(por.cu_q),
+                               _ptr(por.ctx0), _ptr(por.slot), _ptr(por.tseq), por.nseq, por.n, _ptr(state), _ptr(out), _stream()))
+
+
+def rglru_scan(gates: torch.Tensor, u: torch.Tensor, ypre: torch.Tensor, lam: torch.Tensor, c: float, blocks: int, por: Portions,
+               S: torch.Tensor, out: torch.Tensor):
+    lib = load_library()
+    n, channels = u.shape
+    bw = channels // blocks
+    assert n == por.n and gates.dtype == torch.float32 and gates.is_contiguous() and gates.shape == (blocks, n, 2 * bw)
+    assert u.dtype == torch.float32 and u.is_contiguous() and ypre.shape == (n, channels) and ypre.stride(1) == 1
+    assert S.dtype == torch.float32 and S.is_contiguous() and S.shape[1] == channels and lam.numel() == channels
+    assert out.shape == (n, channels) and out.is_contiguous()
+    _check(lib.nvs_rglru_scan(_ptr(gates), _ptr(u), _ptr(ypre), ypre.stride(0), _same(ypre, lam, out), _ptr(lam), c, channels,
+                              blocks, _ptr(por.cu_q), _ptr(por.ctx0), _ptr(por.slot), por.nseq, n, _ptr(S), _ptr(out), _stream()))
+
+
+def ssd_scan(xbc: torch.Tensor, proj: torch.Tensor, dt_col: int, dt_bias, A_log, D, heads: int, P: int, N: int, G: int,
+             por: Portions, S: torch.Tensor, y: torch.Tensor):
+    lib = load_library()
+    n = por.n
+    inner = heads * P
+    assert xbc.dtype == torch.float32 and xbc.is_contiguous() and xbc.shape == (n, inner + 2 * G * N)
+    assert proj.shape[0] == n and proj.stride(1) == 1 and dt_col + heads <= proj.shape[1]
+    assert S.dtype == torch.float32 and S.is_contiguous() and tuple(S.shape[1:]) == (heads, N, P)
+    assert y.dtype == torch.float32 and y.is_contiguous() and y.shape == (n, inner)
+    assert dt_bias.numel() == heads and A_log.numel() == heads and D.numel() == heads
+    _check(lib.nvs_ssd_scan(_ptr(xbc), _ptr(proj), proj.stride(0), dt_col, _same(proj, dt_bias, A_log, D), _ptr(dt_bias),
+                            _ptr(A_log), _ptr(D), heads, P, N, G, _ptr(por.cu_q), _ptr(por.ctx0), _ptr(por.slot), por.nseq, n,
+                            _ptr(S), _ptr(y), _stream()))
+
+
+def gated_group_norm(y: torch.Tensor, z: torch.Tensor, w: torch.Tensor, groups: int, eps: float, out: torch.Tensor):
+    lib = load_library()
+    n, inner = y.shape
+    assert y.dtype == torch.float32 and y.is_contiguous() and z.shape == (n, inner) and z.stride(1) == 1
+    assert w.numel() == inner and out.shape == (n, inner) and out.is_contiguous()
+    _check(lib.nvs_gated_group_norm(_ptr(y), _ptr(z), z.stride(0), _same(z, w, out), _ptr(w), inner, groups, eps, n, _ptr(out),
+                                    _stream()))
+
+
+def knorm_kvstore(k: torch.Tensor, v: torch.Tensor, knorm: torch.Tensor | None, eps: float, G: int, d: int, dv: int,
+                  slots: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor):
+    """k [n, G*d], v [n, G*dv]: column ranges of ONE projection output (same row stride)."""
+    lib = load_library()
+    n = k.shape[0]
+    assert k.shape == (n, G * d) and v.shape == (n, G * dv) and k.stride(1) == 1 and v.stride(1) == 1 and k.stride(0) == v.stride(0)
+    assert slots.dtype == torch.int32 and slots.numel() >= n
+    assert k_cache.is_contiguous() and v_cache.is_contiguous()
+    assert tuple(k_cache.shape[1:]) == (G, d) and tuple(v_cache.shape[1:]) == (G, dv)
+    _check(lib.nvs_knorm_kvstore(_ptr(k), _ptr(v), k.stride(0), _same(k, v, knorm, k_cache, v_cache), _ptr(knorm), eps, G, d, dv,
+                                 _ptr(slots), n, _ptr(k_cache), _ptr(v_cache), _stream()))
+
+
+def window_attn(q: torch.Tensor, qnorm: torch.Tensor | None, eps: float, gate: torch.Tensor | None, k_cache, v_cache,
+                block_tables: torch.Tensor, block_size: int, por: Portions, H: int, G: int, d: int, dv: int, scale: float,
+                window: int, out: torch.Tensor):
+    lib = load_library()
+    n = por.n
+    assert q.shape == (n, H * d) and q.stride(1) == 1 and out.shape == (n, H * dv) and out.is_contiguous()
+    assert gate is None or (gate.shape == (n, H * dv) and gate.stride(1) == 1)
+    assert block_tables.dtype == torch.int32 and block_tables.stride(1) == 1 and block_tables.shape[0] >= por.nseq
+    assert tuple(k_cache.shape[1:]) == (G, d) and tuple(v_cache.shape[1:]) == (G, dv)
+    _check(lib.nvs_window_attn(_ptr(q), q.stride(0), _ptr(qnorm), eps, _ptr(gate), gate.stride(0) if gate is not None else 0,
+                               _same(q, qnorm, gate, k_cache, v_cache, out), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
+                               block_tables.stride(0), block_size, _ptr(por.cu_q), _ptr(por.ctx0), _ptr(por.tseq), por.nseq, n, H,
+                               G, d, dv, scale, window, _ptr(out), _stream()))

@@ -151,6 +151,22 @@ def load_model(model: nn.Module, path: str) -> int:
     if not files:
         raise FileNotFoundError(f"no *.safetensors under {path} (pass dummy_weights=True for random weights)")
     n = 0
+    if hasattr(model, "named_loaders"):
+        # families whose tensors land in fused buffers: the model maps every checkpoint name to a function that copies it
+        # into place. Both directions are checked: a tensor the model does not know, or one it misses, is an error.
+        loaders = model.named_loaders()
+        seen = set()
+        for file in files:
+            with safe_open(file, "pt", "cpu") as f:
+                for name in f.keys():
+                    if name not in loaders:
+                        raise KeyError(f"{file}: tensor {name!r} has no place in {type(model).__name__}")
+                    loaders[name](f.get_tensor(name).to(next(model.parameters()).device))
+                    seen.add(name)
+        missing = sorted(set(loaders) - seen)
+        if missing:
+            raise KeyError(f"checkpoint lacks {len(missing)} tensors, e.g. {missing[:4]}")
+        return len(seen)
     tied = getattr(model, "geo", {}).get("tie", False)
     for file in files:
         with safe_open(file, "pt", "cpu") as f:
