@@ -193,7 +193,7 @@ __global__ void gated_group_norm_kernel(const float* __restrict__ y, const T* __
 extern "C" int nvs_causal_conv(const void* in, int64_t in_stride, int dtype, const void* w, const void* b, int channels, int taps,
                                int act, const int32_t* cu_q, const int32_t* ctx0, const int32_t* slot, const int32_t* tseq, int nseq,
                                int64_t n, float* state, float* out, void* stream) {
-  NVS_REQUIRE(in && w && cu_q && ctx0 && slot && tseq && state && out, "nvs_causal_conv: null argument");
+  NVS_REQUIRE(in && w && cu_q && ctx0 && slot && tseq && (state || taps == 1) && out, "nvs_causal_conv: null argument");
   NVS_REQUIRE(channels > 0 && taps >= 1 && taps <= MAX_TAPS && in_stride >= channels && nseq >= 0 && n >= 0 && (act == 0 || act == 1),
               "nvs_causal_conv: channels %d taps %d (1..%d) stride %lld act %d", channels, taps, MAX_TAPS, (long long)in_stride, act);
   if (n == 0 || nseq == 0) return NVS_OK;

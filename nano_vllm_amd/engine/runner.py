@@ -252,6 +252,7 @@ class _Stage:
 
 
 class ModelRunner:
+    spec = spec_of(None)            # the model family (registry.ModelSpec); set per instance from the configuration
 
     def __init__(self, config: Config, rank: int, event=None):
         """`event` is accepted for signature compatibility with the reference (model_runner.py:17) and unused:

@@ -130,3 +130,87 @@ class FoduzenForCausalLM(nn.Module):
         normed = torch.empty(nrows, x.shape[1], dtype=self.dtype, device=x.device)
         ops_seq.scalar_norm_rows(x, rows, nrows, self.final_norm, self.config.eps, normed)
         return F.linear(normed, self.head)
+
+
+# ---- synthetic checkpoints (tests, benchmarks, dummy weights) -----------------------------------------------------------
+def tensor_shapes(raw: dict) -> dict[str, tuple]:
+    """Checkpoint tensor names -> shapes of a configuration (the parsed config.json)."""
+    W, V = raw["width"], raw["vocab"]
+    out = {"embed": (V, W), "head": (V, W), "final.norm": ()}
+    for i, layer in enumerate(raw["layers"]):
+        p, m = f"l{i}.", layer["mixer"]
+        out[p + "norm1"] = ()
+        if layer["type"] == "rglru":
+            C, nb = m["width"], m["blocks"]
+            bw = C // nb
+            out.update({p + "mix.y": (C, W), p + "mix.y.b": (C,), p + "mix.x": (C, W), p + "mix.x.b": (C,),
+                        p + "mix.conv": (C, m["conv"]), p + "mix.conv.b": (C,), p + "mix.ra": (nb, bw, bw), p + "mix.ra.b": (nb, bw),
+                        p + "mix.ri": (nb, bw, bw), p + "mix.ri.b": (nb, bw), p + "mix.lam": (C,), p + "mix.o": (W, C)})
+        else:
+            le, ri = m["left"], m["right"]
+            H, G, d, dv = le["heads"], le["kv_heads"], le["dim"], le["vdim"]
+            inner, gn = ri["heads"] * ri["vdim"], ri["groups"] * ri["state"]
+            out.update({p + "mix.left.q": (H * d, W), p + "mix.left.q.b": (H * d,), p + "mix.left.k": (G * d, W),
+                        p + "mix.left.k.b": (G * d,), p + "mix.left.v": (G * dv, W), p + "mix.left.v.b": (G * dv,),
+                        p + "mix.left.q.norm": (d,), p + "mix.left.k.norm": (d,), p + "mix.left.g": (H * dv, W),
+                        p + "mix.left.o": (W, H * dv), p + "mix.left.o.b": (W,),
+                        p + "mix.right.in": (2 * inner + 2 * gn + ri["heads"], W), p + "mix.right.conv": (inner + 2 * gn, ri["conv"]),
+                        p + "mix.right.conv.b": (inner + 2 * gn,), p + "mix.right.dt_bias": (ri["heads"],),
+                        p + "mix.right.A_log": (ri["heads"],), p + "mix.right.D": (ri["heads"],), p + "mix.right.norm": (inner,),
+                        p + "mix.right.o": (W, inner), p + "mix.left.out": (W,), p + "mix.right.out": (W,)})
+        if layer.get("mlp") is not None:
+            ff = layer["mlp"]["ff"]
+            out.update({p + "norm2": (), p + "mlp.up": (ff, W), p + "mlp.down": (W, ff), p + "mlp.act": (2,)})
+    return out
+
+
+def random_tensors(raw: dict, seed: int = 0) -> dict[str, torch.Tensor]:
+    """Seeded random bf16 weights in ranges that keep every mechanism alive: decays spread between fast and slow, step
+    sizes around 0.1, matrices scaled by their fan-in."""
+    gen = torch.Generator().manual_seed(seed)
+    out = {}
+    for name, shape in tensor_shapes(raw).items():
+        leaf = name.split(".")[-1]
+        r = torch.randn(shape, generator=gen, dtype=torch.float32)
+        if name.endswith(".lam"):
+            t = -5.0 + 3.0 * torch.rand(shape, generator=gen)                  # a between ~0.6 and ~0.99 at r = 1/2
+        elif leaf == "A_log":
+            t = -2.0 + 2.5 * torch.rand(shape, generator=gen)
+        elif leaf == "dt_bias":
+            t = -3.5 + 2.5 * torch.rand(shape, generator=gen)
+        elif leaf == "D" or leaf in ("norm", "out", "norm1", "norm2") or name == "final.norm":
+            t = 1.0 + 0.1 * r
+        elif leaf == "act":
+            t = 0.5 * r
+        elif leaf == "b" or len(shape) == 1:
+            t = 0.1 * r
+        elif name == "embed":
+            t = 0.05 * r
+        elif leaf in ("conv",):
+            t = 0.5 * r
+        else:
+            t = r / (shape[-1] ** 0.5)
+        out[name] = t.to(torch.bfloat16)
+    return out
+
+
+def write_synthetic_checkpoint(path: str, raw: dict, seed: int = 0) -> str:
+    """config.json + model.safetensors of a random model of the family (no tokenizer: requests are token ids)."""
+    import json
+    import os
+    from safetensors.torch import save_file
+    os.makedirs(path, exist_ok=True)
+    with open(os.path.join(path, "config.json"), "w") as fh:
+        json.dump(raw, fh, indent=1)
+    save_file({k: v.contiguous() for k, v in random_tensors(raw, seed).items()}, os.path.join(path, "model.safetensors"))
+    return path
+
+
+def _init_random(self, seed: int = 0) -> None:
+    loaders = self.named_loaders()
+    dev = self.embed.device
+    for name, t in random_tensors(self.config.raw, seed).items():
+        loaders[name](t.to(dev))
+
+
+FoduzenForCausalLM.init_random = _init_random
