@@ -84,7 +84,82 @@ def parse():
     ap.add_argument("--num-kvcache-blocks", type=int, default=-1)
     ap.add_argument("--kv-cache-dtype", default="bf16", choices=["bf16", "fp8"],
                     help="fp8: opt-in OCP e4m3 KV cache (outside the reference's numerics; never the headline)")
+    ap.add_argument("--compare-families", action="store_true",
+                    help="instead of the headline workload: prefill and decode throughput of the Foduzen family at layer sizes of "
+                         "real models (random weights) beside Qwen3 models of equal width / depth, one JSON line")
+    ap.add_argument("--families", default="foduzen,qwen3", help="with --compare-families: which of the two to run")
+    ap.add_argument("--sizes", default="1k,4k", help="with --compare-families: layer sizes to run (1k, 4k)")
     return ap.parse_args()
+
+
+# ---- model families side by side (--compare-families) ----------------------------------------------------------------------
+def foduzen_config(width: int, ff: int, heads: int, kv_heads: int, layers: int, vocab: int) -> dict:
+    """Layers of a real model's size: 128-wide attention heads with a 1,024-token window, 64-wide state-space heads with 128
+    states, recurrent blocks as wide as the model; parallel and recurrent blocks alternate."""
+    par = {"type": "parallel", "mlp": {"kind": "dense", "ff": ff},
+           "mixer": {"left": {"heads": heads, "kv_heads": kv_heads, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "mask": {"size": 1024}},
+                     "right": {"heads": width // 64, "vdim": 64, "state": 128, "groups": 1, "conv": 4, "norm_groups": 1}}}
+    rec = {"type": "rglru", "mlp": {"kind": "dense", "ff": ff}, "mixer": {"width": width, "blocks": width // 128, "conv": 4}}
+    return {"architecture": "Foduzen", "embedding": {"scale": 1.0}, "layers": [par if i % 2 == 0 else rec for i in range(layers)],
+            "norm": {"eps": 1e-6}, "vocab": vocab, "width": width}
+
+
+FAMILY_SIZES = {   # name: (width, ff, heads, kv heads, layers, the Qwen3 shape of the same width / depth)
+    "1k": (1024, 3072, 16, 8, 4, "qwen3-0.6b-4l"),
+    "4k": (4096, 12288, 32, 8, 2, "qwen3-8b-2l"),
+}
+
+
+def compare_families(args) -> dict:
+    import torch
+    from nano_vllm_amd import SamplingParams
+    from nano_vllm_amd.foduzen import write_synthetic_checkpoint as write_foduzen
+    from nano_vllm_amd.weights import write_synthetic_checkpoint as write_qwen3
+    from nanovllm import LLM
+    vocab = 32768
+    seed(0)
+    pre_prompts = [[randint(0, vocab - 1) for _ in range(2048)] for _ in range(8)]          # one 16,384-token prefill step
+    dec_prompts = [[randint(0, vocab - 1) for _ in range(512)] for _ in range(64)]          # 64 sequences decoding at 512+ context
+    out = {}
+    for size in args.sizes.split(","):
+        width, ff, heads, kv, layers, qname = FAMILY_SIZES[size]
+        for family in args.families.split(","):
+            path = os.path.join(tempfile.gettempdir(), f"nvl_cmp_{family}_{size}")
+            if family == "foduzen":
+                raw = foduzen_config(width, ff, heads, kv, layers, vocab)
+                os.makedirs(path, exist_ok=True)
+                with open(os.path.join(path, "config.json"), "w") as fh:
+                    json.dump(raw, fh)
+            else:
+                write_qwen3(path, qname, with_weights=False, vocab_size=vocab)
+            llm = LLM(path, dummy_weights=True, max_model_len=4096, max_num_batched_tokens=16384, max_num_seqs=64,
+                      enforce_eager=args.eager, gpu_memory_utilization=0.5)
+
+            def run(prompts, n_out):
+                if hasattr(llm, "reset_prefix_cache"):
+                    llm.reset_prefix_cache()
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                llm.generate(prompts, SamplingParams(temperature=0.0, max_tokens=n_out, ignore_eos=True), use_tqdm=False)
+                torch.cuda.synchronize()
+                return time.perf_counter() - t0
+
+            for _ in range(max(args.warmup, 1)):
+                run(pre_prompts, 1)
+                run(dec_prompts, 9)
+            t_pre = min(run(pre_prompts, 1) for _ in range(max(args.steps, 1)))
+            t_d1 = min(run(dec_prompts, 1) for _ in range(max(args.steps, 1)))
+            t_d = min(run(dec_prompts, 129) for _ in range(max(args.steps, 1)))
+            out[f"{family}_{size}"] = {
+                "prefill_tok_s": round(8 * 2048 / t_pre, 1), "prefill_ms": round(t_pre * 1e3, 2),
+                "decode_tok_s": round(64 * 128 / (t_d - t_d1), 1), "decode_ms_per_step": round((t_d - t_d1) / 128 * 1e3, 3),
+                "layers": layers, "width": width}
+            llm.exit()
+            del llm
+            torch.cuda.empty_cache()
+    return {"metric": "family_compare", "unit": "tok/s", "dtype": "bf16", "data": "synthetic", "steps": args.steps,
+            "warmup": args.warmup, "n_gpus": 1, "config": {"prefill": "8 x 2048 tokens, one step", "decode": "64 sequences x 128 tokens "
+            "after 512-token prompts", "vocab": vocab}, "results": out}
 
 
 def workload(num_seqs: int, kind: str = "bench"):
@@ -148,6 +223,11 @@ def main():
     from nano_vllm_amd import build as nvl_build
     if rank == 0 or world == 1:
         nvl_build.build()
+    if args.compare_families:
+        assert world == 1, "--compare-families is a one-GPU measurement"
+        nvl_build.build_seq()
+        print(json.dumps(compare_families(args)), flush=True)
+        return
     dev_index = 0 if share_gpu else local_rank
     torch.cuda.set_device(dev_index)
     if world > 1:

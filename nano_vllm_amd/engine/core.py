@@ -210,7 +210,7 @@ class LLMEngine:
         assert self.scheduler.is_finished(), "reset_prefix_cache() needs an idle engine"
         from .kv_blocks import BlockManager
         bm = self.scheduler.block_manager
-        self.scheduler.block_manager = BlockManager(bm.num_blocks, bm.block_size)
+        self.scheduler.block_manager = BlockManager(bm.num_blocks, bm.block_size, prefix_cache=bm.prefix_cache)
 
     def generate(self, prompts, sampling_params, use_tqdm: bool = True):
         from tqdm.auto import tqdm

@@ -167,17 +167,17 @@ def tensor_shapes(raw: dict) -> dict[str, tuple]:
 def random_tensors(raw: dict, seed: int = 0) -> dict[str, torch.Tensor]:
     """Seeded random bf16 weights in ranges that keep every mechanism alive: decays spread between fast and slow, step
     sizes around 0.1, matrices scaled by their fan-in."""
-    gen = torch.Generator().manual_seed(seed)
+    gen = torch.Generator(device="cpu").manual_seed(seed)
     out = {}
     for name, shape in tensor_shapes(raw).items():
         leaf = name.split(".")[-1]
-        r = torch.randn(shape, generator=gen, dtype=torch.float32)
+        r = torch.randn(shape, generator=gen, dtype=torch.float32, device="cpu")
         if name.endswith(".lam"):
-            t = -5.0 + 3.0 * torch.rand(shape, generator=gen)                  # a between ~0.6 and ~0.99 at r = 1/2
+            t = -5.0 + 3.0 * torch.rand(shape, generator=gen, device="cpu")                  # a between ~0.6 and ~0.99 at r = 1/2
         elif leaf == "A_log":
-            t = -2.0 + 2.5 * torch.rand(shape, generator=gen)
+            t = -2.0 + 2.5 * torch.rand(shape, generator=gen, device="cpu")
         elif leaf == "dt_bias":
-            t = -3.5 + 2.5 * torch.rand(shape, generator=gen)
+            t = -3.5 + 2.5 * torch.rand(shape, generator=gen, device="cpu")
         elif leaf == "D" or leaf in ("norm", "out", "norm1", "norm2") or name == "final.norm":
             t = 1.0 + 0.1 * r
         elif leaf == "act":

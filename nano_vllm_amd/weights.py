@@ -36,6 +36,7 @@ QWEN3_SHAPES = {
     "qwen3-tiny-kv8": (512, 1024, 2, 16, 8, False),       # 8 kv heads: shards down to 1 kv head per rank at TP = 8
     "qwen3-tiny-g5": (512, 768, 2, 10, 2, False),         # G = 5 (Qwen3-14B's 40 / 8): a group size that does not divide 16
     # two full-width layers of the large models (tests: the layer code paths real 8B / 32B widths take)
+    "qwen3-0.6b-4l": (1024, 3072, 4, 16, 8, True),       # four layers of the 0.6B width (bench.py --compare-families)
     "qwen3-8b-2l": (4096, 12288, 2, 32, 8, False),
     "qwen3-14b-2l": (5120, 17408, 2, 40, 8, False),
     "qwen3-32b-2l": (5120, 25600, 2, 64, 8, False),
