@@ -68,7 +68,7 @@ int nvs_rglru_scan(const float* gates, const float* u, const void* ypre, int64_t
 /* State-space-duality recurrence, recurrent form. xbc [n, inner + 2*G*N] 32-bit (x | B | C after convolution + SiLU),
  * dt: column dt_col .. dt_col + heads of proj [n, proj_stride] (`dtype`); dt_bias, A_log, D [heads] (`dtype`). Per head h
  * (group h / (heads / G)), token by token: dt = softplus(dt + dt_bias), S = exp(-exp(A_log) dt) S + dt B x^T,
- * y = S^T C + D x. S [nslots, heads, N, P] 32-bit, advanced. y [n, heads * P] 32-bit. */
+ * y = S^T C + D x. State memory is [nslots, heads, P, N] (n fastest), 32-bit, advanced. y [n, heads * P] 32-bit. */
 int nvs_ssd_scan(const float* xbc, const void* proj, int64_t proj_stride, int64_t dt_col, int dtype, const void* dt_bias,
                  const void* A_log, const void* D, int heads, int P, int N, int G, const int32_t* cu_q, const int32_t* ctx0,
                  const int32_t* slot, int nseq, int64_t n, float* S, float* y, void* stream);
@@ -80,19 +80,26 @@ int nvs_gated_group_norm(const float* y, const void* z, int64_t z_stride, int dt
 
 /* Key norm + paged K/V store. k [n, G, d] / v [n, G, dv] are column ranges of one projection output (row stride `stride`,
  * `dtype`). k is RMS-normed over d with weight knorm [d] (NULL: stored as is). Token t goes to cache slot slots[t] (< 0:
- * skipped). Caches: k_cache [nslots_kv, G, d], v_cache [nslots_kv, G, dv], `dtype`; slot = block * block_size + offset. */
+ * skipped); slot = page * block_size + offset. Caches, `dtype`: k_cache [slot][G][d]; v_cache [page][G][dv][block_size] — values
+ * are kept TRANSPOSED inside a page, so that a column's consecutive tokens are contiguous (the matrix-core attention reads 8 at a
+ * time). */
 int nvs_knorm_kvstore(const void* k, const void* v, int64_t stride, int dtype, const void* knorm, float eps, int G, int d, int dv,
-                      const int32_t* slots, int64_t n, void* k_cache, void* v_cache, void* stream);
+                      int block_size, const int32_t* slots, int64_t n, void* k_cache, void* v_cache, void* stream);
 
 /* Sliding-window softmax attention over the paged cache, one query per token row, any d, dv <= 256.
  * q [n, H, d] (row stride q_stride), RMS-normed per head with qnorm [d] here (NULL: none). Token t of portion s sits at position
  * p = ctx0[s] + (t - cu_q[s]) and sees keys j with 0 <= p - j < window (window <= 0: every j <= p), read through
  * block_tables [nseq, bt_stride]. score = q.k * scale, ordinary softmax in 32-bit. gate (nullable) [n, H*dv] with row stride
- * gate_stride: out *= sigmoid(gate). out [n, H*dv] `dtype`. */
+ * gate_stride: out *= sigmoid(gate). out [n, H*dv] `dtype`.
+ * bf16 with d % 8 == 0 and block_size % 8 == 0 runs on the matrix cores (16 queries per wavefront; the weights enter the
+ * second product as bf16); everything else, and every float32 call, takes the scalar kernel (one wavefront per query). */
 int nvs_window_attn(const void* q, int64_t q_stride, const void* qnorm, float eps, const void* gate, int64_t gate_stride, int dtype,
                     const void* k_cache, const void* v_cache, const int32_t* block_tables, int64_t bt_stride, int block_size,
                     const int32_t* cu_q, const int32_t* ctx0, const int32_t* tseq, int nseq, int64_t n, int H, int G, int d, int dv,
                     float scale, int window, void* out, void* stream);
+
+/* Tests: route bf16 calls through the scalar kernel too (1) or back (0). */
+void nvs_window_attn_force_scalar(int on);
 
 #ifdef __cplusplus
 }

@@ -10,8 +10,8 @@ constexpr int MAX_HEAD = 256;
 // one wavefront per (token, kv head)
 template <typename T>
 __global__ void knorm_kvstore_kernel(const T* __restrict__ k, const T* __restrict__ v, int64_t stride, const T* __restrict__ knorm,
-                                     float eps, int G, int d, int dv, const int32_t* __restrict__ slots, T* __restrict__ k_cache,
-                                     T* __restrict__ v_cache) {
+                                     float eps, int G, int d, int dv, int block_size, const int32_t* __restrict__ slots,
+                                     T* __restrict__ k_cache, T* __restrict__ v_cache) {
   const int64_t t = blockIdx.x;
   const int g = blockIdx.y, lane = threadIdx.x;
   const int64_t slot = slots[t];
@@ -34,8 +34,10 @@ __global__ void knorm_kvstore_kernel(const T* __restrict__ k, const T* __restric
     if (c < d) stf(kc + c, knorm ? kv[i] * r * ldf(knorm + c) : kv[i]);
   }
   const T* vp = v + t * stride + (int64_t)g * dv;
-  T* vc = v_cache + (slot * G + g) * dv;
-  for (int c = lane; c < dv; c += 64) vc[c] = vp[c];
+  // values are kept transposed inside a page, [page][G][dv][block]: the attention kernels read a column's consecutive tokens
+  const int64_t page = slot / block_size, off = slot - page * block_size;
+  T* vc = v_cache + ((page * G + g) * dv) * block_size + off;
+  for (int c = lane; c < dv; c += 64) vc[(int64_t)c * block_size] = vp[c];
 }
 
 // one wavefront per (token, query head). Keys go in rounds of 64 (one per lane): score, running maximum, weights into LDS,
@@ -49,7 +51,7 @@ __global__ void window_attn_kernel(const T* __restrict__ q, int64_t q_stride, co
                                    T* __restrict__ out) {
   __shared__ float qs[MAX_HEAD];
   __shared__ float ps[64];
-  __shared__ int64_t slot_s[64];
+  __shared__ int64_t slot_s[64];                    // element offset of (token, column 0) in the page-transposed V cache
   const int64_t t = blockIdx.x;
   const int h = blockIdx.y, lane = threadIdx.x;
   const int s = tseq[t];
@@ -84,9 +86,11 @@ __global__ void window_attn_kernel(const T* __restrict__ q, int64_t q_stride, co
     const int64_t j = j0 + lane;
     const bool live = j <= pos;
     float sc = -INFINITY;
-    int64_t slot = 0;
+    int64_t slot = 0, voff = 0;
     if (live) {
-      slot = (int64_t)bt[j / block_size] * block_size + j % block_size;
+      const int64_t page = bt[j / block_size], off = j % block_size;
+      slot = page * block_size + off;
+      voff = ((page * G + g) * dv) * block_size + off;
       const T* kp = k_cache + (slot * G + g) * d;
       float dot = 0.f;
       for (int c = 0; c < d; ++c) dot += qs[c] * ldf(kp + c);
@@ -99,7 +103,7 @@ __global__ void window_attn_kernel(const T* __restrict__ q, int64_t q_stride, co
     m = mn;
     __syncthreads();                                  // the previous round's readers are done
     ps[lane] = p;
-    slot_s[lane] = slot;
+    slot_s[lane] = voff;
     __syncthreads();
     const int cnt = (int)((pos - j0 + 1) < 64 ? (pos - j0 + 1) : 64);
 #pragma unroll
@@ -107,7 +111,7 @@ __global__ void window_attn_kernel(const T* __restrict__ q, int64_t q_stride, co
       const int c = lane + 64 * i;
       if (c < dv) {
         float a = acc[i] * alpha;
-        for (int jj = 0; jj < cnt; ++jj) a += ps[jj] * ldf(v_cache + (slot_s[jj] * G + g) * dv + c);
+        for (int jj = 0; jj < cnt; ++jj) a += ps[jj] * ldf(v_cache + slot_s[jj] + (int64_t)c * block_size);
         acc[i] = a;
       }
     }
@@ -127,16 +131,186 @@ __global__ void window_attn_kernel(const T* __restrict__ q, int64_t q_stride, co
   }
 }
 
+
+// ---- bf16 matrix-core form ------------------------------------------------------------------------------------------
+// One wavefront per (16 consecutive queries of a portion, query head); four query tiles per workgroup, no LDS. Everything
+// is computed transposed so that each lane owns ONE query (column l & 15) and the softmax statistics need two shuffles:
+//   S^T[keys x queries] = K Q^T   v_mfma_f32_16x16x32_bf16, A = 16 key rows x 32 of d (16-byte loads from the K cache),
+//                                 B = Q^T (normed, scaled, held in registers for the whole tile)
+//   O^T[dv x queries]  += V^T P^T A = 16 value columns x 32 tokens: 16-byte loads from the page-transposed V cache,
+//                                 B = P^T straight from the S^T accumulators of two key blocks
+// The MFMA's contraction index may be permuted freely as long as both operands agree; the key rows of block kb are the
+// tokens base + 32 (kb / 2) + 8 (i / 4) + 4 (kb % 2) + i % 4, which makes the 8 weights a lane holds after two key blocks
+// the 8 CONSECUTIVE tokens its V load covers. Scores, maxima, sums and O stay 32-bit; the weights enter the second product
+// as bf16, like V. d % 8 == 0, block_size % 8 == 0; d and dv are padded to the template's sizes with zero operands.
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+typedef __attribute__((ext_vector_type(4))) unsigned int u32x4_t;
+
+template <int DK, int DVB>     // d <= 32 DK, dv <= 16 DVB
+__global__ __launch_bounds__(256) void window_attn_mfma_kernel(
+    const bf16_t* __restrict__ q, int64_t q_stride, const bf16_t* __restrict__ qnorm, float eps, const bf16_t* __restrict__ gate,
+    int64_t gate_stride, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+    const int32_t* __restrict__ block_tables, int64_t bt_stride, int block_size, const int32_t* __restrict__ cu_q,
+    const int32_t* __restrict__ ctx0, int nseq, int H, int G, int d, int dv, float scale, int window, bf16_t* __restrict__ out) {
+  const int lane = threadIdx.x & 63, qi = lane & 15, gq = lane >> 4;
+  int tile = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int h = blockIdx.y, g = h / (H / G);
+  int s = 0, len = 0;
+  for (; s < nseq; ++s) {
+    len = cu_q[s + 1] - cu_q[s];
+    const int tiles = (len + 15) >> 4;
+    if (tile < tiles) break;
+    tile -= tiles;
+  }
+  if (s >= nseq) return;                            // (no workgroup barrier below: a wavefront may leave alone)
+  const int rel = tile * 16 + qi;
+  const bool valid_q = rel < len;
+  const int64_t row = (int64_t)cu_q[s] + (valid_q ? rel : len - 1);
+  const int64_t pos = (int64_t)ctx0[s] + rel;
+  const int64_t p_first = (int64_t)ctx0[s] + tile * 16;
+  const int64_t p_last = (int64_t)ctx0[s] + (tile * 16 + 15 < len ? tile * 16 + 15 : len - 1);
+
+  // Q^T operand: lane holds d elements [32 c + 8 gq, + 8) of query qi, normed and scaled
+  bf16x8_t qb[DK];
+  {
+    float qv[DK][8];
+    float ss = 0.f;
+    const bf16_t* qp = q + row * q_stride + (int64_t)h * d;
+#pragma unroll
+    for (int c = 0; c < DK; ++c)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int col = c * 32 + gq * 8 + e;
+        qv[c][e] = col < d ? (float)qp[col] : 0.f;
+        ss += qv[c][e] * qv[c][e];
+      }
+    float r = scale;
+    if (qnorm) {
+      ss += __shfl_xor(ss, 16, 64);
+      ss += __shfl_xor(ss, 32, 64);
+      r *= rsqrtf(ss / (float)d + eps);
+    }
+#pragma unroll
+    for (int c = 0; c < DK; ++c)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int col = c * 32 + gq * 8 + e;
+        const float w = (qnorm && col < d) ? (float)qnorm[col] : 1.f;
+        qb[c][e] = (bf16_t)(qv[c][e] * r * w);
+      }
+  }
+  const int64_t lo = window > 0 ? (p_first - window + 1 > 0 ? p_first - window + 1 : 0) : 0;
+  const int32_t* bt = block_tables + (int64_t)s * bt_stride;
+  float m = -1e30f, lsum = 0.f;
+  f32x4_t oacc[DVB];
+#pragma unroll
+  for (int db = 0; db < DVB; ++db) oacc[db] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  const bf16x8_t zero8 = __builtin_bit_cast(bf16x8_t, u32x4_t{0u, 0u, 0u, 0u});
+
+  for (int64_t j0 = lo & ~(int64_t)31; j0 <= p_last; j0 += 64) {
+    // ---- S^T for 64 tokens: 4 key blocks
+    f32x4_t sacc[4];
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb) {
+      sacc[kb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      const int64_t j = j0 + (kb >> 1) * 32 + (qi >> 2) * 8 + (kb & 1) * 4 + (qi & 3);      // the token of this lane's A row
+      const bool have = j <= p_last;
+      const bf16_t* kp = k_cache;
+      if (have) kp += (((int64_t)bt[j / block_size] * block_size + j % block_size) * G + g) * d + gq * 8;
+#pragma unroll
+      for (int c = 0; c < DK; ++c) {
+        bf16x8_t a = zero8;
+        if (have && c * 32 + gq * 8 < d) a = *(const bf16x8_t*)(kp + c * 32);
+        sacc[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qb[c], sacc[kb], 0, 0, 0);
+      }
+    }
+    // ---- mask, running maximum, weights (this lane: query qi, tokens 32 (kb/2) + 8 gq + 4 (kb%2) + r)
+    float mx = m;
+    bool ok[4][4];
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int64_t j = j0 + (kb >> 1) * 32 + gq * 8 + (kb & 1) * 4 + r;
+        ok[kb][r] = valid_q && j <= pos && (window <= 0 || pos - j < window);
+        if (ok[kb][r]) mx = fmaxf(mx, sacc[kb][r]);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float alpha = __expf(m - mx);
+    m = mx;
+    lsum *= alpha;
+    bf16x8_t pb[2];
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float p = ok[kb][r] ? __expf(sacc[kb][r] - mx) : 0.f;
+        lsum += p;
+        pb[kb >> 1][(kb & 1) * 4 + r] = (bf16_t)p;
+      }
+#pragma unroll
+    for (int db = 0; db < DVB; ++db) oacc[db] *= alpha;
+    // ---- O^T += V^T P^T: two groups of 32 tokens
+#pragma unroll
+    for (int mg = 0; mg < 2; ++mg) {
+      const int64_t jb = j0 + mg * 32 + gq * 8;                                             // 8 consecutive tokens, one page
+      const bool have = jb <= p_last;
+      const bf16_t* vp = v_cache;
+      if (have) vp += (((int64_t)bt[jb / block_size] * G + g) * dv) * block_size + jb % block_size;
+#pragma unroll
+      for (int db = 0; db < DVB; ++db) {
+        const int col = db * 16 + qi;
+        bf16x8_t a = zero8;
+        if (have && col < dv) a = *(const bf16x8_t*)(vp + (int64_t)col * block_size);
+        oacc[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb[mg], oacc[db], 0, 0, 0);
+      }
+    }
+  }
+  lsum += __shfl_xor(lsum, 16, 64);
+  lsum += __shfl_xor(lsum, 32, 64);
+  if (!valid_q) return;
+  const float inv = 1.f / lsum;
+  bf16_t* op = out + ((int64_t)row * H + h) * dv;
+  const bf16_t* gp = gate ? gate + row * gate_stride + (int64_t)h * dv : nullptr;
+#pragma unroll
+  for (int db = 0; db < DVB; ++db)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int c = db * 16 + gq * 4 + r;
+      if (c < dv) {
+        float o = oacc[db][r] * inv;
+        if (gp) o *= 1.f / (1.f + expf(-(float)gp[c]));
+        op[c] = (bf16_t)o;
+      }
+    }
+}
+
+template <int DK, int DVB>
+void launch_mfma(const void* q, int64_t q_stride, const void* qnorm, float eps, const void* gate, int64_t gate_stride,
+                 const void* k_cache, const void* v_cache, const int32_t* block_tables, int64_t bt_stride, int block_size,
+                 const int32_t* cu_q, const int32_t* ctx0, int nseq, int64_t n, int H, int G, int d, int dv, float scale, int window,
+                 void* out, hipStream_t stream) {
+  const int64_t tiles = n / 16 + nseq;              // an upper bound: every portion may end with a partial tile
+  window_attn_mfma_kernel<DK, DVB><<<dim3((unsigned)((tiles + 3) / 4), H), dim3(256), 0, stream>>>(
+      (const bf16_t*)q, q_stride, (const bf16_t*)qnorm, eps, (const bf16_t*)gate, gate_stride, (const bf16_t*)k_cache,
+      (const bf16_t*)v_cache, block_tables, bt_stride, block_size, cu_q, ctx0, nseq, H, G, d, dv, scale, window, (bf16_t*)out);
+}
 }  // namespace
 
+static int g_force_scalar = 0;
+/* tests: 1 routes bf16 calls through the scalar kernel as well */
+extern "C" void nvs_window_attn_force_scalar(int on) { g_force_scalar = on; }
+
 extern "C" int nvs_knorm_kvstore(const void* k, const void* v, int64_t stride, int dtype, const void* knorm, float eps, int G, int d,
-                                 int dv, const int32_t* slots, int64_t n, void* k_cache, void* v_cache, void* stream) {
+                                 int dv, int block_size, const int32_t* slots, int64_t n, void* k_cache, void* v_cache, void* stream) {
   NVS_REQUIRE(k && v && slots && k_cache && v_cache, "nvs_knorm_kvstore: null argument");
-  NVS_REQUIRE(G > 0 && G <= 65535 && d > 0 && d <= MAX_HEAD && dv > 0 && dv <= MAX_HEAD && n >= 0, "nvs_knorm_kvstore: G %d d %d dv %d", G,
-              d, dv);
+  NVS_REQUIRE(G > 0 && G <= 65535 && d > 0 && d <= MAX_HEAD && dv > 0 && dv <= MAX_HEAD && n >= 0 && block_size > 0,
+              "nvs_knorm_kvstore: G %d d %d dv %d", G, d, dv);
   if (n == 0) return NVS_OK;
   NVS_DISPATCH(dtype, knorm_kvstore_kernel<T><<<dim3((unsigned)n, G), dim3(64), 0, (hipStream_t)stream>>>(
-                          (const T*)k, (const T*)v, stride, (const T*)knorm, eps, G, d, dv, slots, (T*)k_cache, (T*)v_cache));
+                          (const T*)k, (const T*)v, stride, (const T*)knorm, eps, G, d, dv, block_size, slots, (T*)k_cache, (T*)v_cache));
   return nvs_check_launch("nvs_knorm_kvstore");
 }
 
@@ -148,6 +322,17 @@ extern "C" int nvs_window_attn(const void* q, int64_t q_stride, const void* qnor
   NVS_REQUIRE(H > 0 && H <= 65535 && G > 0 && H % G == 0 && d > 0 && d <= MAX_HEAD && dv > 0 && dv <= MAX_HEAD && block_size > 0 && n >= 0,
               "nvs_window_attn: H %d G %d d %d dv %d block %d", H, G, d, dv, block_size);
   if (n == 0 || nseq == 0) return NVS_OK;
+  if (dtype == NVS_BF16 && d % 8 == 0 && block_size % 8 == 0 && !g_force_scalar) {
+    const int dk = d <= 64 ? 2 : (d <= 128 ? 4 : 8), dvb = dv <= 64 ? 4 : (dv <= 128 ? 8 : 16);
+#define NVS_MFMA_CASE(DK, DVB)                                                                                                  \
+  if (dk == DK && dvb == DVB)                                                                                                   \
+    launch_mfma<DK, DVB>(q, q_stride, qnorm, eps, gate, gate_stride, k_cache, v_cache, block_tables, bt_stride, block_size, cu_q, \
+                         ctx0, nseq, n, H, G, d, dv, scale, window, out, (hipStream_t)stream);
+    NVS_MFMA_CASE(2, 4) NVS_MFMA_CASE(2, 8) NVS_MFMA_CASE(2, 16) NVS_MFMA_CASE(4, 4) NVS_MFMA_CASE(4, 8) NVS_MFMA_CASE(4, 16)
+    NVS_MFMA_CASE(8, 4) NVS_MFMA_CASE(8, 8) NVS_MFMA_CASE(8, 16)
+#undef NVS_MFMA_CASE
+    return nvs_check_launch("nvs_window_attn (matrix cores)");
+  }
   NVS_DISPATCH(dtype, window_attn_kernel<T><<<dim3((unsigned)n, H), dim3(64), 0, (hipStream_t)stream>>>(
                           (const T*)q, q_stride, (const T*)qnorm, eps, (const T*)gate, gate_stride, (const T*)k_cache, (const T*)v_cache,
                           block_tables, bt_stride, block_size, cu_q, ctx0, tseq, H, G, d, dv, scale, window, (T*)out));

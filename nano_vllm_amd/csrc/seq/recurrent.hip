@@ -104,68 +104,90 @@ __global__ void rglru_scan_kernel(const float* __restrict__ gates, const float* 
 }
 
 // ---- state-space-duality recurrence -------------------------------------------------------------------------------
-// one workgroup per (portion, head): blockDim = (P, NG); thread (p, g) keeps S[n, p] for n = g, g + NG, ... in registers.
-// Per token: S <- dA S + dt B[n] x[p]; partial y[p] = sum over own n of S C[n]; partials meet in LDS.
+// One workgroup per (portion, head), P * NG threads: thread (p, g) = (tid / NG, tid % NG) keeps the 16 state entries
+// S[p][16 g .. 16 g + 15] in registers (state memory is [heads][P][N], n fastest: a thread's entries are contiguous).
+// Tokens go in rounds of TB: the round's x | B | C | dt are staged in LDS by all threads (the NEXT round's global loads
+// are issued before the current round is computed), then every token costs 16 x (2 FMA + 1 MUL) per thread, LDS
+// reads that vectorise, and log2(NG) shuffles for y[p] = sum_n S C: the NG threads of a p are neighbouring lanes.
 constexpr int SSD_R = 16;      // state entries per thread
-constexpr int SSD_TB = 4;      // tokens per LDS round
+constexpr int SSD_PF = 32;     // staged values per thread and round, at most
 
 template <typename T>
 __global__ void ssd_scan_kernel(const float* __restrict__ xbc, const T* __restrict__ proj, int64_t proj_stride, int64_t dt_col,
                                 const T* __restrict__ dt_bias, const T* __restrict__ A_log, const T* __restrict__ Dp, int heads,
-                                int P, int N, int G, const int32_t* __restrict__ cu_q, const int32_t* __restrict__ ctx0,
-                                const int32_t* __restrict__ slot, float* __restrict__ S, float* __restrict__ y) {
-  extern __shared__ float part[];                   // [SSD_TB][NG][P]
-  const int s = blockIdx.y, h = blockIdx.x;
-  const int p = threadIdx.x, g = threadIdx.y, NG = blockDim.y;
+                                int P, int N, int G, int NG, int TB, const int32_t* __restrict__ cu_q,
+                                const int32_t* __restrict__ ctx0, const int32_t* __restrict__ slot, float* __restrict__ S,
+                                float* __restrict__ y) {
+  extern __shared__ __attribute__((aligned(16))) float lds[];   // [TB][per]: x (P) | B (NP) | C (NP) | dt, NP = 16 NG, zero padded
+  const int s = blockIdx.y, h = blockIdx.x, tid = threadIdx.x, nthreads = blockDim.x;
+  const int g = tid & (NG - 1), p = tid / NG;
   const int64_t q0 = cu_q[s], q1 = cu_q[s + 1];
   if (q1 <= q0) return;
+  const int NP = NG * SSD_R, P4 = (P + 3) & ~3, per = P4 + 2 * NP + 4;    // every part starts 16-byte aligned
   const int inner = heads * P, grp = h / (heads / G);
   const int64_t row = inner + 2 * G * N;
   const float A = -expf(ldf(A_log + h)), Dh = ldf(Dp + h), dtb = ldf(dt_bias + h);
-  float* Sh = S + (((int64_t)slot[s] * heads + h) * N) * P;
+  float* Sh = S + (((int64_t)slot[s] * heads + h) * P + p) * N + g * SSD_R;
   float st[SSD_R];
   const bool fresh = ctx0[s] == 0;
 #pragma unroll
-  for (int r = 0; r < SSD_R; ++r) {
-    const int nn = g + r * NG;
-    st[r] = (!fresh && nn < N) ? Sh[(int64_t)nn * P + p] : 0.f;
-  }
-  for (int64_t tb = q0; tb < q1; tb += SSD_TB) {
-    const int cnt = (int)((q1 - tb) < SSD_TB ? (q1 - tb) : SSD_TB);
+  for (int r = 0; r < SSD_R; ++r) st[r] = (!fresh && g * SSD_R + r < N) ? Sh[r] : 0.f;
+
+  float pf[SSD_PF];
+  auto fetch = [&](int64_t tb) {                    // global -> registers, for the round that starts at token tb
+    const int total = (int)((q1 - tb) < TB ? (q1 - tb) : TB) * per;
+#pragma unroll
+    for (int i = 0; i < SSD_PF; ++i) {
+      const int idx = tid + i * nthreads;
+      float v = 0.f;
+      if (idx < total) {
+        const int k = idx / per, c = idx - k * per;
+        const int64_t t = tb + k;
+        if (c < P4) {
+          if (c < P) v = xbc[t * row + h * P + c];
+        } else if (c < P4 + NP) {
+          if (c - P4 < N) v = xbc[t * row + inner + grp * N + (c - P4)];
+        } else if (c < P4 + 2 * NP) {
+          if (c - P4 - NP < N) v = xbc[t * row + inner + G * N + grp * N + (c - P4 - NP)];
+        } else if (c == P4 + 2 * NP) {
+          v = softplusf_(ldf(proj + t * proj_stride + dt_col + h) + dtb);
+        }
+      }
+      pf[i] = v;
+    }
+  };
+  fetch(q0);
+  for (int64_t tb = q0; tb < q1; tb += TB) {
+    const int cnt = (int)((q1 - tb) < TB ? (q1 - tb) : TB);
+    __syncthreads();                                // the previous round's readers are done
+#pragma unroll
+    for (int i = 0; i < SSD_PF; ++i) {
+      const int idx = tid + i * nthreads;
+      if (idx < cnt * per) lds[idx] = pf[i];
+    }
+    __syncthreads();
+    if (tb + TB < q1) fetch(tb + TB);
     for (int k = 0; k < cnt; ++k) {
-      const int64_t t = tb + k;
-      const float* rowp = xbc + t * row;
-      const float dt = softplusf_(ldf(proj + t * proj_stride + dt_col + h) + dtb);
+      const float* tp = lds + k * per;
+      const float dt = tp[P4 + 2 * NP];
       const float dA = expf(A * dt);
-      const float xv = rowp[h * P + p];
-      const float* Bp = rowp + inner + grp * N;
-      const float* Cp = rowp + inner + G * N + grp * N;
+      const float xv = tp[p];
+      const float* Bp = (const float*)__builtin_assume_aligned(tp + P4 + g * SSD_R, 16);
+      const float* Cp = (const float*)__builtin_assume_aligned(Bp + NP, 16);
+      const float dx = dt * xv;
       float acc = 0.f;
 #pragma unroll
       for (int r = 0; r < SSD_R; ++r) {
-        const int nn = g + r * NG;
-        if (nn < N) {
-          st[r] = dA * st[r] + (dt * Bp[nn]) * xv;
-          acc += st[r] * Cp[nn];
-        }
+        st[r] = dA * st[r] + Bp[r] * dx;
+        acc += st[r] * Cp[r];
       }
-      part[(k * NG + g) * P + p] = acc;
+      for (int o = NG >> 1; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
+      if (g == 0) y[(tb + k) * inner + h * P + p] = acc + Dh * xv;
     }
-    __syncthreads();
-    // thread (p, g) finishes token g of the round (NG >= SSD_TB is guaranteed by the launcher, or loops)
-    for (int k = g; k < cnt; k += NG) {
-      float acc = 0.f;
-      for (int gg = 0; gg < NG; ++gg) acc += part[(k * NG + gg) * P + p];
-      const int64_t t = tb + k;
-      y[t * inner + h * P + p] = acc + Dh * xbc[t * row + h * P + p];
-    }
-    __syncthreads();
   }
 #pragma unroll
-  for (int r = 0; r < SSD_R; ++r) {
-    const int nn = g + r * NG;
-    if (nn < N) Sh[(int64_t)nn * P + p] = st[r];
-  }
+  for (int r = 0; r < SSD_R; ++r)
+    if (g * SSD_R + r < N) Sh[r] = st[r];
 }
 
 // ---- gate, then group RMS norm ------------------------------------------------------------------------------------
@@ -237,17 +259,17 @@ extern "C" int nvs_ssd_scan(const float* xbc, const void* proj, int64_t proj_str
   NVS_REQUIRE(heads > 0 && G > 0 && heads % G == 0 && P > 0 && P <= 256 && N > 0 && nseq >= 0 && nseq <= 65535,
               "nvs_ssd_scan: heads %d groups %d head size %d state %d", heads, G, P, N);
   if (n == 0 || nseq == 0) return NVS_OK;
-  int ng = 1024 / P;
-  if (ng > N) ng = N;
-  NVS_REQUIRE(ng * SSD_R >= N, "nvs_ssd_scan: state %d x head size %d exceeds one workgroup's registers", N, P);
-  // no more rows of threads than needed to hold the state, but at least enough to spread the per-round reduction
-  int need = (N + SSD_R - 1) / SSD_R;
-  if (need < SSD_TB) need = SSD_TB < ng ? SSD_TB : ng;
-  ng = need;
-  const size_t lds = (size_t)SSD_TB * ng * P * sizeof(float);
-  NVS_DISPATCH(dtype, ssd_scan_kernel<T><<<dim3(heads, (unsigned)nseq), dim3(P, ng), lds, (hipStream_t)stream>>>(
-                          xbc, (const T*)proj, proj_stride, dt_col, (const T*)dt_bias, (const T*)A_log, (const T*)D, heads, P, N, G, cu_q,
-                          ctx0, slot, S, y));
+  int ng = 1;
+  while (ng * SSD_R < N) ng <<= 1;                  // a power of two: the threads of one p reduce by lane shuffles
+  NVS_REQUIRE(ng <= 64 && (int64_t)P * ng <= 1024, "nvs_ssd_scan: state %d x head size %d exceeds one workgroup's registers", N, P);
+  const int threads = P * ng, per = ((P + 3) & ~3) + 2 * ng * SSD_R + 4;
+  int tb = SSD_PF * threads / per;                  // what the staging registers hold
+  if (tb > 16) tb = 16;
+  NVS_REQUIRE(tb >= 1, "nvs_ssd_scan: head size %d with state %d cannot be staged", P, N);
+  const size_t lds = (size_t)tb * per * sizeof(float);
+  NVS_DISPATCH(dtype, ssd_scan_kernel<T><<<dim3(heads, (unsigned)nseq), dim3(threads), lds, (hipStream_t)stream>>>(
+                          xbc, (const T*)proj, proj_stride, dt_col, (const T*)dt_bias, (const T*)A_log, (const T*)D, heads, P, N, G, ng, tb,
+                          cu_q, ctx0, slot, S, y));
   return nvs_check_launch("nvs_ssd_scan");
 }
 

@@ -48,7 +48,7 @@ class WindowAttention(nn.Module):
         self.scale, self.window, self.eps, self.block_size = float(scale), int(window), eps, block_size
         self.q_norm = _param(dim) if qk_norm else None
         self.k_norm = _param(dim) if qk_norm else None
-        self.k_cache = self.v_cache = None            # [pages * block_size, G, d] / [..., G, dv], injected by the runner
+        self.k_cache = self.v_cache = None            # [pages * block_size, G, d] / [..., G, dv] (values page-transposed), from the runner
 
     @property
     def widths(self) -> tuple[int, int, int, int]:
@@ -61,7 +61,8 @@ class WindowAttention(nn.Module):
 
     def forward(self, q, k, v, gate) -> torch.Tensor:
         ctx = get_context()
-        ops_seq.knorm_kvstore(k, v, self.k_norm, self.eps, self.G, self.d, self.dv, ctx.slot_mapping, self.k_cache, self.v_cache)
+        ops_seq.knorm_kvstore(k, v, self.k_norm, self.eps, self.G, self.d, self.dv, self.block_size, ctx.slot_mapping, self.k_cache,
+                              self.v_cache)
         out = torch.empty(q.shape[0], self.H * self.dv, dtype=q.dtype, device=q.device)
         ops_seq.window_attn(q, self.q_norm, self.eps, gate, self.k_cache, self.v_cache, ctx.block_tables, self.block_size,
                             ctx.portions, self.H, self.G, self.d, self.dv, self.scale, self.window, out)
@@ -87,7 +88,7 @@ class SSDMixer(nn.Module):
         return 2 * self.inner + 2 * self.groups * self.N + self.heads
 
     def state_shapes(self) -> dict:
-        return {"conv_state": (self.taps - 1, self.channels), "rec_state": (self.heads, self.N, self.P)}
+        return {"conv_state": (self.taps - 1, self.channels), "rec_state": (self.heads, self.P, self.N)}
 
     def forward(self, proj: torch.Tensor, col0: int) -> torch.Tensor:
         """`proj`: the fused projection output; this mixer's columns start at col0."""

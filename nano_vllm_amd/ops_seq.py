@@ -29,7 +29,8 @@ SIGNATURES = {
     "nvs_rglru_scan": (c_int, [_P, _P, _P, _L, _I, _P, _F, _I, _I, _P, _P, _P, _I, _L, _P, _P, _P]),
     "nvs_ssd_scan": (c_int, [_P, _P, _L, _L, _I, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _I, _L, _P, _P, _P]),
     "nvs_gated_group_norm": (c_int, [_P, _P, _L, _I, _P, _I, _I, _F, _L, _P, _P]),
-    "nvs_knorm_kvstore": (c_int, [_P, _P, _L, _I, _P, _F, _I, _I, _I, _P, _L, _P, _P, _P]),
+    "nvs_knorm_kvstore": (c_int, [_P, _P, _L, _I, _P, _F, _I, _I, _I, _I, _P, _L, _P, _P, _P]),
+    "nvs_window_attn_force_scalar": (None, [_I]),
     "nvs_window_attn": (c_int, [_P, _L, _P, _F, _P, _L, _I, _P, _P, _P, _L, _I, _P, _P, _P, _I, _L, _I, _I, _I, _I, _F, _I,
                                 _P, _P]),
 }
@@ -53,6 +54,8 @@ def load_library() -> ctypes.CDLL:
         fn.restype, fn.argtypes = restype, argtypes
     if lib.nvs_abi_version() != ABI_VERSION:
         raise NvsError(f"libnvl_seq.so ABI version {lib.nvs_abi_version()} != binding version {ABI_VERSION}; rebuild")
+    if os.environ.get("NVL_ATTN_SCALAR") == "1":      # A/B switch: bf16 windowed attention on the scalar kernel too
+        lib.nvs_window_attn_force_scalar(1)
     _lib = lib
     return lib
 
@@ -171,7 +174,7 @@ def ssd_scan(xbc: torch.Tensor, proj: torch.Tensor, dt_col: int, dt_bias, A_log,
     inner = heads * P
     assert xbc.dtype == torch.float32 and xbc.is_contiguous() and xbc.shape == (n, inner + 2 * G * N)
     assert proj.shape[0] == n and proj.stride(1) == 1 and dt_col + heads <= proj.shape[1]
-    assert S.dtype == torch.float32 and S.is_contiguous() and tuple(S.shape[1:]) == (heads, N, P)
+    assert S.dtype == torch.float32 and S.is_contiguous() and tuple(S.shape[1:]) == (heads, P, N)
     assert y.dtype == torch.float32 and y.is_contiguous() and y.shape == (n, inner)
     assert dt_bias.numel() == heads and A_log.numel() == heads and D.numel() == heads
     _check(lib.nvs_ssd_scan(_ptr(xbc), _ptr(proj), proj.stride(0), dt_col, _same(proj, dt_bias, A_log, D), _ptr(dt_bias),
@@ -189,8 +192,10 @@ def gated_group_norm(y: torch.Tensor, z: torch.Tensor, w: torch.Tensor, groups: 
 
 
 def knorm_kvstore(k: torch.Tensor, v: torch.Tensor, knorm: torch.Tensor | None, eps: float, G: int, d: int, dv: int,
-                  slots: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor):
-    """k [n, G*d], v [n, G*dv]: column ranges of ONE projection output (same row stride)."""
+                  block_size: int, slots: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor):
+    """k [n, G*d], v [n, G*dv]: column ranges of ONE projection output (same row stride). v_cache has the shape
+    [pages * block_size, G, dv] but is laid out [page][G][dv][block_size] (see include/nvl_seq.h)."""
+    assert k_cache.shape[0] % block_size == 0
     lib = load_library()
     n = k.shape[0]
     assert k.shape == (n, G * d) and v.shape == (n, G * dv) and k.stride(1) == 1 and v.stride(1) == 1 and k.stride(0) == v.stride(0)
@@ -198,7 +203,7 @@ def knorm_kvstore(k: torch.Tensor, v: torch.Tensor, knorm: torch.Tensor | None, 
     assert k_cache.is_contiguous() and v_cache.is_contiguous()
     assert tuple(k_cache.shape[1:]) == (G, d) and tuple(v_cache.shape[1:]) == (G, dv)
     _check(lib.nvs_knorm_kvstore(_ptr(k), _ptr(v), k.stride(0), _same(k, v, knorm, k_cache, v_cache), _ptr(knorm), eps, G, d, dv,
-                                 _ptr(slots), n, _ptr(k_cache), _ptr(v_cache), _stream()))
+                                 block_size, _ptr(slots), n, _ptr(k_cache), _ptr(v_cache), _stream()))
 
 
 def window_attn(q: torch.Tensor, qnorm: torch.Tensor | None, eps: float, gate: torch.Tensor | None, k_cache, v_cache,

@@ -171,7 +171,7 @@ def test_state_space_recurrence_against_the_token_loop(heads, P, N, G):
             gg = h // (heads // G)
             S[h] = torch.exp(-torch.exp(A_log[h].double()) * dt[t, h]) * S[h] + dt[t, h] * torch.outer(B[t, gg], x[t, h])
             want[t, h] = S[h].T @ Cm[t, gg] + D[h].double() * x[t, h]
-    state = torch.full((2, heads, N, P), 5.0, device="cuda")
+    state = torch.full((2, heads, P, N), 5.0, device="cuda")
     outs = []
     for lo, hi in ((0, 1), (1, 3), (3, 50), (50, 90)):
         y = torch.empty(hi - lo, inner, device="cuda")
@@ -179,7 +179,7 @@ def test_state_space_recurrence_against_the_token_loop(heads, P, N, G):
                          portions([hi - lo], [lo], [1]), state, y)
         outs.append(y)
     close(torch.cat(outs).view(T, heads, P), want, 2e-5, "outputs")
-    close(state[1], S, 2e-5, "final state")
+    close(state[1].transpose(1, 2), S, 2e-5, "final state")      # kept [heads, P, N]
 
 
 def test_gate_then_group_norm():
@@ -210,7 +210,7 @@ def _attend(q, k, v, H, G, d, dv, scale, window, block, lens, order, qn=None, kn
     kc = torch.full((total, G, d), 77.0, device="cuda", dtype=dtype)
     vc = torch.full((total, G, dv), 77.0, device="cuda", dtype=dtype)
     kv = dev(torch.cat([k, v], 1).to(dtype))
-    ops_seq.knorm_kvstore(kv[:, :G * d], kv[:, G * d:], None if kn is None else dev(kn.to(dtype)), eps, G, d, dv,
+    ops_seq.knorm_kvstore(kv[:, :G * d], kv[:, G * d:], None if kn is None else dev(kn.to(dtype)), eps, G, d, dv, block,
                           torch.tensor(slots, dtype=torch.int32, device="cuda"), kc, vc)
     out = torch.empty(sum(lens), H * dv, device="cuda", dtype=dtype)
     ops_seq.window_attn(dev(q.to(dtype)), None if qn is None else dev(qn.to(dtype)), eps, None if gate is None else dev(gate.to(dtype)),
@@ -236,23 +236,33 @@ def _plain_attention(q, k, v, H, G, d, dv, scale, window, qn=None, kn=None, gate
 
 @pytest.mark.parametrize("H,G,d,dv,window,block", [(4, 2, 32, 48, 20, 16), (3, 3, 64, 128, 64, 64), (8, 1, 16, 16, 1, 16),
                                                    (2, 2, 80, 200, 0, 32), (6, 2, 128, 64, 33, 48)])
-def test_windowed_attention_against_the_plain_loop(H, G, d, dv, window, block):
+@pytest.mark.parametrize("dtype,path", [(torch.float32, "scalar"), (torch.bfloat16, "matrix"), (torch.bfloat16, "scalar")])
+def test_windowed_attention_against_the_plain_loop(H, G, d, dv, window, block, dtype, path):
+    """float32 takes the one-query-per-wavefront kernel; bfloat16 the matrix-core kernel (16 queries per wavefront), or the
+    scalar one when forced — the path head sizes outside the matrix-core kernel's reach take."""
+    from nano_vllm_amd import ops_seq
     g = torch.Generator().manual_seed(H * d)
     lens = [70, 5, 129]
     T = sum(lens)
-    q, k, v = torch.randn(T, H * d, generator=g), torch.randn(T, G * d, generator=g), torch.randn(T, G * dv, generator=g)
-    qn, kn, gate = 1 + 0.2 * torch.randn(d, generator=g), 1 + 0.2 * torch.randn(d, generator=g), torch.randn(T, H * dv, generator=g)
+    rnd = lambda *shape: torch.randn(*shape, generator=g).to(dtype).float()
+    q, k, v = rnd(T, H * d), rnd(T, G * d), rnd(T, G * dv)
+    qn, kn, gate = (1 + 0.2 * rnd(d)).to(dtype).float(), (1 + 0.2 * rnd(d)).to(dtype).float(), rnd(T, H * dv)
     order = torch.randperm(sum(-(-L // block) for L in lens) + 3, generator=g).tolist()      # scattered pages
-    got = _attend(q, k, v, H, G, d, dv, 0.4, window, block, lens, order, qn, kn, gate)
+    ops_seq.load_library().nvs_window_attn_force_scalar(int(path == "scalar"))
+    try:
+        got = _attend(q, k, v, H, G, d, dv, 0.4, window, block, lens, order, qn, kn, gate, dtype=dtype)
+    finally:
+        ops_seq.load_library().nvs_window_attn_force_scalar(0)
     o = 0
     for L in lens:
         want = _plain_attention(q[o:o + L], k[o:o + L], v[o:o + L], H, G, d, dv, 0.4, window, qn, kn, gate[o:o + L])
-        close(got[o:o + L], want, 1e-5, f"sequence of {L}")
+        close(got[o:o + L], want, 1e-5 if dtype == torch.float32 else 2e-2, f"sequence of {L}")
         o += L
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("window,block", [(96, 64), (50, 16), (64, 64), (65, 32)])
-def test_a_standout_key_just_inside_and_just_outside_the_window(window, block):
+def test_a_standout_key_just_inside_and_just_outside_the_window(window, block, dtype):
     """One key carries a score far above the rest and a value nobody else has: the query `window - 1` tokens later must
     return that value, the next query must not see it at all — at page borders as elsewhere."""
     H = G = 1
@@ -264,20 +274,21 @@ def test_a_standout_key_just_inside_and_just_outside_the_window(window, block):
         k[hot, 0] = 30.0
         q[:, 0] = 30.0
         v[hot, 3] = 1.0
-        got = _attend(q, k, v, H, G, d, dv, 1.0, window, block, [T], list(range(-(-T // block))))[:, 3].cpu()
+        got = _attend(q, k, v, H, G, d, dv, 1.0, window, block, [T], list(range(-(-T // block))), dtype=dtype)[:, 3].float().cpu()
         last = hot + window - 1
-        assert got[hot:last + 1].min() > 0.999, (hot, "inside the window")
+        assert got[hot:last + 1].min() > 0.99, (hot, "inside the window")
         assert got[last + 1:].abs().max() == 0 and (hot == 0 or got[:hot].abs().max() == 0), (hot, "outside the window")
 
 
-def test_a_far_key_among_hundreds_without_a_window():
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_a_far_key_among_hundreds_without_a_window(dtype):
     H, G, d, dv, T = 2, 1, 32, 32, 900
     g = torch.Generator().manual_seed(9)
     q, k, v = 0.01 * torch.randn(T, H * d, generator=g), 0.01 * torch.randn(T, d, generator=g), torch.zeros(T, dv)
     k[2, 1], v[2, 0] = 25.0, 1.0
     q[:, 1], q[:, d + 1] = 25.0, 25.0
-    got = _attend(q, k, v, H, G, d, dv, 1.0, 0, 64, [T], list(range(15))[::-1]).cpu()
-    assert got[2:, 0].min() > 0.999 and got[2:, dv].min() > 0.999 and got[:2].abs().max() == 0
+    got = _attend(q, k, v, H, G, d, dv, 1.0, 0, 64, [T], list(range(15))[::-1], dtype=dtype).float().cpu()
+    assert got[2:, 0].min() > 0.99 and got[2:, dv].min() > 0.999 and got[:2].abs().max() == 0
 
 
 # ---------------------------------------------------------------------------------------------- the engine
@@ -316,7 +327,7 @@ def rel(got, want, scale):
     return float(np.sqrt((d ** 2).mean(-1)).max() / scale)
 
 
-TOL = {"float32": 5e-5, "bfloat16": 3e-2}
+TOL = {"float32": 5e-5, "bfloat16": 4e-2}      # bf16: logits themselves are bf16 (2^-9 of their size), on top of the layers
 
 
 @pytest.mark.parametrize("variant", [0, 1, 2])
