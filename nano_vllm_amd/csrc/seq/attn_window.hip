@@ -147,36 +147,45 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 typedef __attribute__((ext_vector_type(4))) unsigned int u32x4_t;
 
-template <int DK, int DVB>     // d <= 32 DK, dv <= 16 DVB
+template <int DK, int DVB, int QT>     // d <= 32 DK, dv <= 16 DVB, QT tiles of 16 queries per wavefront (they share every K / V load)
 __global__ __launch_bounds__(256) void window_attn_mfma_kernel(
     const bf16_t* __restrict__ q, int64_t q_stride, const bf16_t* __restrict__ qnorm, float eps, const bf16_t* __restrict__ gate,
     int64_t gate_stride, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int32_t* __restrict__ block_tables, int64_t bt_stride, int block_size, const int32_t* __restrict__ cu_q,
-    const int32_t* __restrict__ ctx0, int nseq, int H, int G, int d, int dv, float scale, int window, bf16_t* __restrict__ out) {
+    const int32_t* __restrict__ ctx0, int nseq, int H, int G, int d, int dv, float scale, int window, int bs_shift,
+    bf16_t* __restrict__ out) {
+  constexpr int QW = 16 * QT;                       // queries per wavefront
   const int lane = threadIdx.x & 63, qi = lane & 15, gq = lane >> 4;
   int tile = blockIdx.x * 4 + (threadIdx.x >> 6);
   const int h = blockIdx.y, g = h / (H / G);
   int s = 0, len = 0;
   for (; s < nseq; ++s) {
     len = cu_q[s + 1] - cu_q[s];
-    const int tiles = (len + 15) >> 4;
+    const int tiles = (len + QW - 1) / QW;
     if (tile < tiles) break;
     tile -= tiles;
   }
   if (s >= nseq) return;                            // (no workgroup barrier below: a wavefront may leave alone)
-  const int rel = tile * 16 + qi;
-  const bool valid_q = rel < len;
-  const int64_t row = (int64_t)cu_q[s] + (valid_q ? rel : len - 1);
-  const int64_t pos = (int64_t)ctx0[s] + rel;
-  const int64_t p_first = (int64_t)ctx0[s] + tile * 16;
-  const int64_t p_last = (int64_t)ctx0[s] + (tile * 16 + 15 < len ? tile * 16 + 15 : len - 1);
+  // positions fit 32 bits (the engine's tables do); page and offset of a token by shift and mask when pages are a power of two
+  const int c0 = ctx0[s];
+  const int p_first = c0 + tile * QW;
+  const int p_last = c0 + (tile * QW + QW - 1 < len ? tile * QW + QW - 1 : len - 1);
+  const int bs_mask = block_size - 1;
 
-  // Q^T operand: lane holds d elements [32 c + 8 gq, + 8) of query qi, normed and scaled
-  bf16x8_t qb[DK];
-  {
+  // Q^T operands: lane holds d elements [32 c + 8 gq, + 8) of query qi of each tile, normed and scaled
+  bf16x8_t qb[QT][DK];
+  bool valid_q[QT];
+  int64_t row[QT];
+  int pos[QT];
+#pragma unroll
+  for (int t = 0; t < QT; ++t) {
+    const int rel = tile * QW + t * 16 + qi;
+    valid_q[t] = rel < len;
+    row[t] = (int64_t)cu_q[s] + (valid_q[t] ? rel : len - 1);
+    pos[t] = c0 + rel;
     float qv[DK][8];
     float ss = 0.f;
-    const bf16_t* qp = q + row * q_stride + (int64_t)h * d;
+    const bf16_t* qp = q + row[t] * q_stride + (int64_t)h * d;
 #pragma unroll
     for (int c = 0; c < DK; ++c)
 #pragma unroll
@@ -197,105 +206,159 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(
       for (int e = 0; e < 8; ++e) {
         const int col = c * 32 + gq * 8 + e;
         const float w = (qnorm && col < d) ? (float)qnorm[col] : 1.f;
-        qb[c][e] = (bf16_t)(qv[c][e] * r * w);
+        qb[t][c][e] = (bf16_t)(qv[c][e] * r * w);
       }
   }
-  const int64_t lo = window > 0 ? (p_first - window + 1 > 0 ? p_first - window + 1 : 0) : 0;
+  const int lo = window > 0 ? (p_first - window + 1 > 0 ? p_first - window + 1 : 0) : 0;
   const int32_t* bt = block_tables + (int64_t)s * bt_stride;
-  float m = -1e30f, lsum = 0.f;
-  f32x4_t oacc[DVB];
+  float m[QT], lsum[QT];
+  f32x4_t oacc[QT][DVB];
 #pragma unroll
-  for (int db = 0; db < DVB; ++db) oacc[db] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  for (int t = 0; t < QT; ++t) {
+    m[t] = -1e30f;
+    lsum[t] = 0.f;
+#pragma unroll
+    for (int db = 0; db < DVB; ++db) oacc[t][db] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  }
   const bf16x8_t zero8 = __builtin_bit_cast(bf16x8_t, u32x4_t{0u, 0u, 0u, 0u});
 
-  for (int64_t j0 = lo & ~(int64_t)31; j0 <= p_last; j0 += 64) {
-    // ---- S^T for 64 tokens: 4 key blocks
-    f32x4_t sacc[4];
+  for (int j0 = lo & ~31; j0 <= p_last; j0 += 64) {
+    // every query of the wavefront sees all 64 tokens of the round: no masks (most rounds of a long window)
+    const bool interior = j0 + 63 <= p_first && (window <= 0 || c0 + tile * QW + QW - 1 - j0 < window);
+    // ---- S^T for 64 tokens: 4 key blocks, every K fragment feeds all QT tiles
+    f32x4_t sacc[QT][4];
 #pragma unroll
     for (int kb = 0; kb < 4; ++kb) {
-      sacc[kb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-      const int64_t j = j0 + (kb >> 1) * 32 + (qi >> 2) * 8 + (kb & 1) * 4 + (qi & 3);      // the token of this lane's A row
+#pragma unroll
+      for (int t = 0; t < QT; ++t) sacc[t][kb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      const int j = j0 + (kb >> 1) * 32 + (qi >> 2) * 8 + (kb & 1) * 4 + (qi & 3);          // the token of this lane's A row
       const bool have = j <= p_last;
       const bf16_t* kp = k_cache;
-      if (have) kp += (((int64_t)bt[j / block_size] * block_size + j % block_size) * G + g) * d + gq * 8;
+      if (have) {
+        const int pg = bs_shift >= 0 ? j >> bs_shift : j / block_size;
+        const int off = bs_shift >= 0 ? j & bs_mask : j - pg * block_size;
+        kp += (((int64_t)bt[pg] * block_size + off) * G + g) * d + gq * 8;
+      }
 #pragma unroll
       for (int c = 0; c < DK; ++c) {
         bf16x8_t a = zero8;
         if (have && c * 32 + gq * 8 < d) a = *(const bf16x8_t*)(kp + c * 32);
-        sacc[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qb[c], sacc[kb], 0, 0, 0);
+#pragma unroll
+        for (int t = 0; t < QT; ++t) sacc[t][kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qb[t][c], sacc[t][kb], 0, 0, 0);
       }
     }
-    // ---- mask, running maximum, weights (this lane: query qi, tokens 32 (kb/2) + 8 gq + 4 (kb%2) + r)
-    float mx = m;
-    bool ok[4][4];
+    // ---- mask, running maximum, weights (this lane: query qi of tile t, tokens 32 (kb/2) + 8 gq + 4 (kb%2) + r)
+    bf16x8_t pb[QT][2];
 #pragma unroll
-    for (int kb = 0; kb < 4; ++kb)
+    for (int t = 0; t < QT; ++t) {
+      float mx = m[t];
+      unsigned okbits = 0xffffu;                     // bit 4 kb + r: the token is visible to this lane's query
+      if (!interior) {
+        okbits = 0u;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int64_t j = j0 + (kb >> 1) * 32 + gq * 8 + (kb & 1) * 4 + r;
-        ok[kb][r] = valid_q && j <= pos && (window <= 0 || pos - j < window);
-        if (ok[kb][r]) mx = fmaxf(mx, sacc[kb][r]);
-      }
-    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float alpha = __expf(m - mx);
-    m = mx;
-    lsum *= alpha;
-    bf16x8_t pb[2];
+        for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
-    for (int kb = 0; kb < 4; ++kb)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const float p = ok[kb][r] ? __expf(sacc[kb][r] - mx) : 0.f;
-        lsum += p;
-        pb[kb >> 1][(kb & 1) * 4 + r] = (bf16_t)p;
+          for (int r = 0; r < 4; ++r) {
+            const int j = j0 + (kb >> 1) * 32 + gq * 8 + (kb & 1) * 4 + r;
+            const bool ok = valid_q[t] && j <= pos[t] && (window <= 0 || pos[t] - j < window);
+            okbits |= ok ? (1u << (kb * 4 + r)) : 0u;
+          }
       }
 #pragma unroll
-    for (int db = 0; db < DVB; ++db) oacc[db] *= alpha;
-    // ---- O^T += V^T P^T: two groups of 32 tokens
+      for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (okbits & (1u << (kb * 4 + r))) mx = fmaxf(mx, sacc[t][kb][r]);
+      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float alpha = __expf(m[t] - mx);
+      m[t] = mx;
+      float ls = lsum[t] * alpha;
+#pragma unroll
+      for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float p = (okbits & (1u << (kb * 4 + r))) ? __expf(sacc[t][kb][r] - mx) : 0.f;
+          ls += p;
+          pb[t][kb >> 1][(kb & 1) * 4 + r] = (bf16_t)p;
+        }
+      lsum[t] = ls;
+      if (__ballot(alpha != 1.f) != 0ull) {          // the maximum moved for some query of the tile
+#pragma unroll
+        for (int db = 0; db < DVB; ++db) oacc[t][db] *= alpha;
+      }
+    }
+    // ---- O^T += V^T P^T: two groups of 32 tokens, every V fragment feeds all QT tiles
 #pragma unroll
     for (int mg = 0; mg < 2; ++mg) {
-      const int64_t jb = j0 + mg * 32 + gq * 8;                                             // 8 consecutive tokens, one page
+      const int jb = j0 + mg * 32 + gq * 8;                                                 // 8 consecutive tokens, one page
       const bool have = jb <= p_last;
       const bf16_t* vp = v_cache;
-      if (have) vp += (((int64_t)bt[jb / block_size] * G + g) * dv) * block_size + jb % block_size;
+      if (have) {
+        const int pg = bs_shift >= 0 ? jb >> bs_shift : jb / block_size;
+        const int off = bs_shift >= 0 ? jb & bs_mask : jb - pg * block_size;
+        vp += (((int64_t)bt[pg] * G + g) * dv) * block_size + off;
+      }
 #pragma unroll
       for (int db = 0; db < DVB; ++db) {
         const int col = db * 16 + qi;
         bf16x8_t a = zero8;
         if (have && col < dv) a = *(const bf16x8_t*)(vp + (int64_t)col * block_size);
-        oacc[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb[mg], oacc[db], 0, 0, 0);
+#pragma unroll
+        for (int t = 0; t < QT; ++t) oacc[t][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb[t][mg], oacc[t][db], 0, 0, 0);
       }
     }
   }
-  lsum += __shfl_xor(lsum, 16, 64);
-  lsum += __shfl_xor(lsum, 32, 64);
-  if (!valid_q) return;
-  const float inv = 1.f / lsum;
-  bf16_t* op = out + ((int64_t)row * H + h) * dv;
-  const bf16_t* gp = gate ? gate + row * gate_stride + (int64_t)h * dv : nullptr;
 #pragma unroll
-  for (int db = 0; db < DVB; ++db)
+  for (int t = 0; t < QT; ++t) {
+    float ls = lsum[t];
+    ls += __shfl_xor(ls, 16, 64);
+    ls += __shfl_xor(ls, 32, 64);
+    if (!valid_q[t]) continue;
+    const float inv = 1.f / ls;
+    bf16_t* op = out + ((int64_t)row[t] * H + h) * dv;
+    const bf16_t* gp = gate ? gate + row[t] * gate_stride + (int64_t)h * dv : nullptr;
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const int c = db * 16 + gq * 4 + r;
-      if (c < dv) {
-        float o = oacc[db][r] * inv;
-        if (gp) o *= 1.f / (1.f + expf(-(float)gp[c]));
-        op[c] = (bf16_t)o;
+    for (int db = 0; db < DVB; ++db)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int c = db * 16 + gq * 4 + r;
+        if (c < dv) {
+          float o = oacc[t][db][r] * inv;
+          if (gp) o *= 1.f / (1.f + expf(-(float)gp[c]));
+          op[c] = (bf16_t)o;
+        }
       }
-    }
+  }
 }
 
+template <int DK, int DVB, int QT>
+void launch_mfma_qt(const void* q, int64_t q_stride, const void* qnorm, float eps, const void* gate, int64_t gate_stride,
+                    const void* k_cache, const void* v_cache, const int32_t* block_tables, int64_t bt_stride, int block_size,
+                    const int32_t* cu_q, const int32_t* ctx0, int nseq, int64_t n, int H, int G, int d, int dv, float scale, int window,
+                    void* out, hipStream_t stream) {
+  const int64_t tiles = n / (16 * QT) + nseq;       // an upper bound: every portion may end with a partial tile
+  int bs_shift = -1;
+  for (int b = 0; b < 31; ++b)
+    if ((1 << b) == block_size) bs_shift = b;
+  window_attn_mfma_kernel<DK, DVB, QT><<<dim3((unsigned)((tiles + 3) / 4), H), dim3(256), 0, stream>>>(
+      (const bf16_t*)q, q_stride, (const bf16_t*)qnorm, eps, (const bf16_t*)gate, gate_stride, (const bf16_t*)k_cache,
+      (const bf16_t*)v_cache, block_tables, bt_stride, block_size, cu_q, ctx0, nseq, H, G, d, dv, scale, window, bs_shift, (bf16_t*)out);
+}
+
+// Long portions (prefill) put two tiles of 16 queries on a wavefront: half the K / V bytes through the vector cache per
+// MFMA; steps of short portions (decoding) keep one tile, which gives more wavefronts.
 template <int DK, int DVB>
 void launch_mfma(const void* q, int64_t q_stride, const void* qnorm, float eps, const void* gate, int64_t gate_stride,
                  const void* k_cache, const void* v_cache, const int32_t* block_tables, int64_t bt_stride, int block_size,
                  const int32_t* cu_q, const int32_t* ctx0, int nseq, int64_t n, int H, int G, int d, int dv, float scale, int window,
                  void* out, hipStream_t stream) {
-  const int64_t tiles = n / 16 + nseq;              // an upper bound: every portion may end with a partial tile
-  window_attn_mfma_kernel<DK, DVB><<<dim3((unsigned)((tiles + 3) / 4), H), dim3(256), 0, stream>>>(
-      (const bf16_t*)q, q_stride, (const bf16_t*)qnorm, eps, (const bf16_t*)gate, gate_stride, (const bf16_t*)k_cache,
-      (const bf16_t*)v_cache, block_tables, bt_stride, block_size, cu_q, ctx0, nseq, H, G, d, dv, scale, window, (bf16_t*)out);
+  if (n >= 32ll * nseq)
+    launch_mfma_qt<DK, DVB, 2>(q, q_stride, qnorm, eps, gate, gate_stride, k_cache, v_cache, block_tables, bt_stride, block_size, cu_q,
+                               ctx0, nseq, n, H, G, d, dv, scale, window, out, stream);
+  else
+    launch_mfma_qt<DK, DVB, 1>(q, q_stride, qnorm, eps, gate, gate_stride, k_cache, v_cache, block_tables, bt_stride, block_size, cu_q,
+                               ctx0, nseq, n, H, G, d, dv, scale, window, out, stream);
 }
 }  // namespace
 

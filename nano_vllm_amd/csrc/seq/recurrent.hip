@@ -106,14 +106,13 @@ __global__ void rglru_scan_kernel(const float* __restrict__ gates, const float* 
 // ---- state-space-duality recurrence -------------------------------------------------------------------------------
 // One workgroup per (portion, head), P * NG threads: thread (p, g) = (tid / NG, tid % NG) keeps the 16 state entries
 // S[p][16 g .. 16 g + 15] in registers (state memory is [heads][P][N], n fastest: a thread's entries are contiguous).
-// Tokens go in rounds of TB: the round's x | B | C | dt are staged in LDS by all threads (the NEXT round's global loads
-// are issued before the current round is computed), then every token costs 16 x (2 FMA + 1 MUL) per thread, LDS
+// Tokens go in rounds of TB: the round's x | B | C | dt | decay are staged in LDS by all threads, then every token costs 16 x (2 FMA + 1 MUL) per thread, LDS
 // reads that vectorise, and log2(NG) shuffles for y[p] = sum_n S C: the NG threads of a p are neighbouring lanes.
 constexpr int SSD_R = 16;      // state entries per thread
-constexpr int SSD_PF = 32;     // staged values per thread and round, at most
+constexpr int SSD_U = 6;       // staging loads a thread keeps in flight
 
 template <typename T>
-__global__ void ssd_scan_kernel(const float* __restrict__ xbc, const T* __restrict__ proj, int64_t proj_stride, int64_t dt_col,
+__global__ __launch_bounds__(1024) void ssd_scan_kernel(const float* __restrict__ xbc, const T* __restrict__ proj, int64_t proj_stride, int64_t dt_col,
                                 const T* __restrict__ dt_bias, const T* __restrict__ A_log, const T* __restrict__ Dp, int heads,
                                 int P, int N, int G, int NG, int TB, const int32_t* __restrict__ cu_q,
                                 const int32_t* __restrict__ ctx0, const int32_t* __restrict__ slot, float* __restrict__ S,
@@ -133,44 +132,53 @@ __global__ void ssd_scan_kernel(const float* __restrict__ xbc, const T* __restri
 #pragma unroll
   for (int r = 0; r < SSD_R; ++r) st[r] = (!fresh && g * SSD_R + r < N) ? Sh[r] : 0.f;
 
-  float pf[SSD_PF];
-  auto fetch = [&](int64_t tb) {                    // global -> registers, for the round that starts at token tb
-    const int total = (int)((q1 - tb) < TB ? (q1 - tb) : TB) * per;
-#pragma unroll
-    for (int i = 0; i < SSD_PF; ++i) {
-      const int idx = tid + i * nthreads;
-      float v = 0.f;
-      if (idx < total) {
-        const int k = idx / per, c = idx - k * per;
-        const int64_t t = tb + k;
-        if (c < P4) {
-          if (c < P) v = xbc[t * row + h * P + c];
-        } else if (c < P4 + NP) {
-          if (c - P4 < N) v = xbc[t * row + inner + grp * N + (c - P4)];
-        } else if (c < P4 + 2 * NP) {
-          if (c - P4 - NP < N) v = xbc[t * row + inner + G * N + grp * N + (c - P4 - NP)];
-        } else if (c == P4 + 2 * NP) {
-          v = softplusf_(ldf(proj + t * proj_stride + dt_col + h) + dtb);
-        }
-      }
-      pf[i] = v;
-    }
-  };
-  fetch(q0);
+  const float* xh = xbc + h * P;
+  const float* Bg = xbc + inner + grp * N;
+  const float* Cg = Bg + G * N;
   for (int64_t tb = q0; tb < q1; tb += TB) {
     const int cnt = (int)((q1 - tb) < TB ? (q1 - tb) : TB);
     __syncthreads();                                // the previous round's readers are done
+    // stage the round: other workgroups of the CU compute meanwhile (LDS and registers leave room for several)
+    // (SSD_U independent loads per thread are in flight before the first LDS store)
+    const int total = cnt * per;
+    for (int base = tid; base < total; base += SSD_U * nthreads) {
+      float v[SSD_U];
 #pragma unroll
-    for (int i = 0; i < SSD_PF; ++i) {
-      const int idx = tid + i * nthreads;
-      if (idx < cnt * per) lds[idx] = pf[i];
+      for (int u = 0; u < SSD_U; ++u) {
+        const int idx = base + u * nthreads;
+        v[u] = 0.f;
+        if (idx < total) {
+          const int k = idx / per, c = idx - k * per;
+          const int64_t t = tb + k;
+          if (c < P) {
+            v[u] = xh[t * row + c];
+          } else if (c >= P4 && c < P4 + NP) {
+            if (c - P4 < N) v[u] = Bg[t * row + (c - P4)];
+          } else if (c >= P4 + NP && c < P4 + 2 * NP) {
+            if (c - P4 - NP < N) v[u] = Cg[t * row + (c - P4 - NP)];
+          } else if (c >= P4 + 2 * NP && c <= P4 + 2 * NP + 1) {
+            v[u] = ldf(proj + t * proj_stride + dt_col + h);
+          }
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < SSD_U; ++u) {
+        const int idx = base + u * nthreads;
+        if (idx < total) {
+          const int c = idx % per;
+          float w = v[u];
+          if (c >= P4 + 2 * NP && c <= P4 + 2 * NP + 1) {          // step size, and the decay it gives
+            w = softplusf_(w + dtb);
+            if (c == P4 + 2 * NP + 1) w = expf(A * w);
+          }
+          lds[idx] = w;
+        }
+      }
     }
     __syncthreads();
-    if (tb + TB < q1) fetch(tb + TB);
     for (int k = 0; k < cnt; ++k) {
       const float* tp = lds + k * per;
-      const float dt = tp[P4 + 2 * NP];
-      const float dA = expf(A * dt);
+      const float dt = tp[P4 + 2 * NP], dA = tp[P4 + 2 * NP + 1];
       const float xv = tp[p];
       const float* Bp = (const float*)__builtin_assume_aligned(tp + P4 + g * SSD_R, 16);
       const float* Cp = (const float*)__builtin_assume_aligned(Bp + NP, 16);
@@ -263,9 +271,7 @@ extern "C" int nvs_ssd_scan(const float* xbc, const void* proj, int64_t proj_str
   while (ng * SSD_R < N) ng <<= 1;                  // a power of two: the threads of one p reduce by lane shuffles
   NVS_REQUIRE(ng <= 64 && (int64_t)P * ng <= 1024, "nvs_ssd_scan: state %d x head size %d exceeds one workgroup's registers", N, P);
   const int threads = P * ng, per = ((P + 3) & ~3) + 2 * ng * SSD_R + 4;
-  int tb = SSD_PF * threads / per;                  // what the staging registers hold
-  if (tb > 16) tb = 16;
-  NVS_REQUIRE(tb >= 1, "nvs_ssd_scan: head size %d with state %d cannot be staged", P, N);
+  const int tb = 16;                                // tokens per LDS round
   const size_t lds = (size_t)tb * per * sizeof(float);
   NVS_DISPATCH(dtype, ssd_scan_kernel<T><<<dim3(heads, (unsigned)nseq), dim3(threads), lds, (hipStream_t)stream>>>(
                           xbc, (const T*)proj, proj_stride, dt_col, (const T*)dt_bias, (const T*)A_log, (const T*)D, heads, P, N, G, ng, tb,
