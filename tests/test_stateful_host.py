@@ -1,0 +1,175 @@
+"""Host side of stateful model families, no GPU: state slots, page tables that grow by portions, the caller-fixed step of
+the scheduler, the prefix cache switch, the model registry and the Foduzen configuration / checkpoint naming."""
+import json
+import os
+import types
+
+import pytest
+import torch
+
+from nano_vllm_amd.engine.kv_blocks import BlockManager
+from nano_vllm_amd.engine.sched import Scheduler
+from nano_vllm_amd.engine.seq import Sequence, SequenceStatus
+from nano_vllm_amd.engine.state_slots import StateSlotManager
+
+
+def fdz_raw():
+    par = {"type": "parallel", "mlp": {"kind": "dense", "ff": 24},
+           "mixer": {"left": {"heads": 4, "kv_heads": 2, "dim": 8, "vdim": 16, "scale": 0.3, "mask": {"size": 5}},
+                     "right": {"heads": 2, "vdim": 8, "state": 4, "groups": 1, "conv": 3, "norm_groups": 2}}}
+    rec = {"type": "rglru", "mlp": None, "mixer": {"width": 24, "blocks": 3, "conv": 2}}
+    return {"architecture": "Foduzen", "embedding": {"scale": 2.0}, "layers": [rec, par], "norm": {"eps": 1e-5}, "vocab": 31, "width": 16}
+
+
+def sched_config(stateful=True, blocks=8, block_size=16, seqs=2, budget=64):
+    from nano_vllm_amd.foduzen import FoduzenConfig
+    hf = FoduzenConfig(fdz_raw()) if stateful else None
+    return types.SimpleNamespace(max_num_seqs=seqs, max_num_batched_tokens=budget, eos=-1, kvcache_block_size=block_size,
+                                 num_kvcache_blocks=blocks, hf_config=hf)
+
+
+def test_state_slots_lowest_first_and_reused():
+    m = StateSlotManager(3)
+    a, b, c = Sequence([1]), Sequence([2]), Sequence([3])
+    assert [m.allocate(s) for s in (a, b, c)] == [0, 1, 2] and not m.can_allocate()
+    m.release(b)
+    assert b.state_slot == -1 and m.num_free == 1
+    d = Sequence([4])
+    assert m.allocate(d) == 1
+    m.release(a), m.release(c), m.release(d)
+    m.release(d)                                   # releasing twice is harmless
+    assert m.num_free == 3
+    with pytest.raises(AssertionError):
+        m.allocate(a), m.allocate(a)
+
+
+def test_block_manager_without_prefix_cache_never_shares_and_extends_by_portions():
+    Sequence.block_size = 4
+    bm = BlockManager(6, 4, prefix_cache=False)
+    a, b = Sequence([7] * 9), Sequence([7] * 9)                    # identical prompts
+    assert bm.can_allocate(a) == 0
+    bm.allocate(a, 0)
+    a.num_scheduled_tokens = 9
+    bm.hash_blocks(a)
+    assert bm.can_allocate(b) == 0 and not bm.hash_to_block_id      # nothing to find
+    bm.allocate(b, 0)
+    assert not set(a.block_table) & set(b.block_table) and bm.num_free == 0
+    bm.deallocate(a)
+    c = Sequence([1, 2])
+    assert bm.blocks_to_extend(c, 2) == 1 and bm.can_extend(c, 2)
+    bm.extend(c, 2)
+    gen = c.table_gen
+    assert len(c.block_table) == 1 and gen > 0
+    for t in range(3, 11):
+        c.append_token(t)
+    assert bm.blocks_to_extend(c, 10) == 2
+    bm.extend(c, 10)
+    assert len(c.block_table) == 3 and c.table_gen == gen and bm.num_free == 0
+    assert not bm.can_extend(c, 13)
+    Sequence.block_size = 256
+
+
+def test_caller_fixed_steps_admit_grow_and_retire():
+    Sequence.block_size = 16
+    s = Scheduler(sched_config(blocks=4, seqs=2))
+    assert s.stateful and not s.block_manager.prefix_cache
+    a, b = Sequence(list(range(20))), Sequence([5])
+    batch = s.schedule_portions([(a, 3), (b, 1)])
+    assert batch == [a, b] and (a.state_slot, b.state_slot) == (0, 1) and len(a.block_table) == 1
+    assert a.num_scheduled_tokens == 3 and a.status is SequenceStatus.RUNNING
+    s.finish_portions(batch)
+    assert a.num_cached_tokens == 3 and b.num_cached_tokens == 1
+    batch = s.schedule_portions([(a, 17)])                          # b sits this step out
+    assert len(a.block_table) == 2
+    s.finish_portions(batch)
+    c = Sequence([1] * 40)
+    with pytest.raises(RuntimeError, match="state slot"):
+        s.schedule_portions([(c, 1)])
+    s.retire(b)
+    assert b.state_slot == -1 and not b.block_table
+    with pytest.raises(RuntimeError, match="KV pool"):
+        s.schedule_portions([(c, 40)])                              # 3 pages needed, 2 free
+    s.retire(a)
+    s.retire(c)
+    assert s.block_manager.num_free == 4 and s.state_slots.num_free == 2 and s.is_finished()
+    Sequence.block_size = 256
+
+
+def test_scheduler_of_a_stateful_model_ties_slots_to_pages():
+    """generate()'s own scheduling: a slot with the pages at admission, both back at the end or on preemption."""
+    Sequence.block_size = 16
+    s = Scheduler(sched_config(blocks=3, seqs=2, budget=64))
+    from nano_vllm_amd.api import SamplingParams
+    seqs = [Sequence([1] * 15, SamplingParams(temperature=0, max_tokens=30, ignore_eos=True)) for _ in range(3)]
+    for q in seqs:
+        s.add(q)
+    batch, prefill = s.schedule()
+    assert prefill and batch == seqs[:2] and [q.state_slot for q in seqs] == [0, 1, -1]      # max_num_seqs
+    s.postprocess(batch, [9, 9], True)
+    steps = preempted = 0
+    orig = s.preempt
+    s.preempt = lambda q: (orig(q), globals().__setitem__("_p", q))[0]
+    while not s.is_finished() and steps < 400:
+        batch, prefill = s.schedule()
+        for q in list(s.waiting):
+            assert q.state_slot == -1 and not q.block_table
+        for q in batch:
+            assert q.state_slot >= 0 and q.block_table
+        s.postprocess(batch, [9] * len(batch), prefill)
+        steps += 1
+    assert s.is_finished() and s.state_slots.num_free == 2 and s.block_manager.num_free == 3
+    assert all(q.num_completion_tokens == 30 for q in seqs)
+    Sequence.block_size = 256
+
+
+def test_registry_reads_both_config_layouts(tmp_path):
+    from nano_vllm_amd.registry import REGISTRY, architecture_of, resolve, spec_of
+    (tmp_path / "config.json").write_text(json.dumps(fdz_raw()))
+    spec, cfg = resolve(str(tmp_path))
+    assert spec.stateful and spec.block_multiple == 16 and "float32" in spec.dtypes
+    assert cfg.vocab_size == 31 and cfg.hidden_size == 16 and cfg.num_hidden_layers == 2 and spec_of(cfg) is spec
+    assert architecture_of({"architectures": ["Qwen3ForCausalLM"]}) == "Qwen3ForCausalLM"
+    assert not REGISTRY["Qwen3ForCausalLM"].stateful and REGISTRY["Qwen3ForCausalLM"].block_multiple == 256
+    (tmp_path / "config.json").write_text(json.dumps({"architecture": "Nothing"}))
+    with pytest.raises(ValueError, match="unsupported"):
+        resolve(str(tmp_path))
+    bad = fdz_raw()
+    bad["layers"][0]["type"] = "lstm"
+    (tmp_path / "config.json").write_text(json.dumps(bad))
+    with pytest.raises(ValueError, match="mixer type"):
+        resolve(str(tmp_path))
+
+
+def test_config_checks_follow_the_family(tmp_path):
+    from nano_vllm_amd.api import Config
+    (tmp_path / "config.json").write_text(json.dumps(fdz_raw()))
+    c = Config(str(tmp_path), kvcache_block_size=48, dtype="fp32")
+    assert c.dtype == "float32" and c.hf_config.architecture == "Foduzen"
+    with pytest.raises(AssertionError):
+        Config(str(tmp_path), kvcache_block_size=40)
+    with pytest.raises(AssertionError):
+        Config(str(tmp_path), tensor_parallel_size=2)
+
+
+def test_checkpoint_names_and_the_models_loaders_agree():
+    """Every tensor the synthetic checkpoint writes has a loader in the model and the other way round, shapes included."""
+    from nano_vllm_amd.foduzen import FoduzenConfig, FoduzenForCausalLM, random_tensors, tensor_shapes
+    raw = fdz_raw()
+    model = FoduzenForCausalLM(FoduzenConfig(raw), torch.float32, block_size=16)
+    loaders = model.named_loaders()
+    shapes = tensor_shapes(raw)
+    assert set(loaders) == set(shapes)
+    tensors = random_tensors(raw, seed=3)
+    with torch.no_grad():
+        for name, t in tensors.items():
+            assert tuple(t.shape) == tuple(shapes[name]) and t.dtype == torch.bfloat16
+            loaders[name](t)
+    mix = model.layers[1].mix
+    q = mix.attn.widths[0]
+    assert torch.equal(mix.in_w[:q], tensors["l1.mix.left.q"].float())
+    assert torch.equal(mix.in_b[q + sum(mix.attn.widths[1:]):], torch.zeros(mix.ssd.in_width))      # no bias on that part
+    rec = model.layers[0].mix
+    assert torch.equal(rec.gate_w[1, :, :8], tensors["l0.mix.ra"][1].float().T)
+    assert model.layers[0].mlp is None and model.layers[0].norm2 is None
+    with pytest.raises(AssertionError):
+        loaders["embed"](torch.zeros(3, 3))
