@@ -98,7 +98,8 @@ int nvs_window_attn(const void* q, int64_t q_stride, const void* qnorm, float ep
                     const int32_t* cu_q, const int32_t* ctx0, const int32_t* tseq, int nseq, int64_t n, int H, int G, int d, int dv,
                     float scale, int window, void* out, void* stream);
 
-/* Tests: route bf16 calls through the scalar kernel too (1) or back (0). */
+/* Tests and A/B runs: 1 routes bf16 calls through the scalar kernel too; 2 keeps the matrix-core kernel but without sharing
+ * K / V tiles through LDS; 0 restores the defaults. */
 void nvs_window_attn_force_scalar(int on);
 
 #ifdef __cplusplus

@@ -146,6 +146,7 @@ __global__ void window_attn_kernel(const T* __restrict__ q, int64_t q_stride, co
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 typedef __attribute__((ext_vector_type(4))) unsigned int u32x4_t;
+int g_no_lds = 0;          // tests / A-B: 1 keeps every wavefront on its own operand loads (no LDS sharing)
 
 template <int DK, int DVB, int QT>     // d <= 32 DK, dv <= 16 DVB, QT tiles of 16 queries per wavefront (they share every K / V load)
 __global__ __launch_bounds__(256) void window_attn_mfma_kernel(
@@ -332,15 +333,241 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(
   }
 }
 
+// ---- the same, with the K / V tiles of a round shared through LDS ------------------------------------------------------
+// A workgroup of four wavefronts serves ONE kv head: `hw` query heads of its group times 4 / hw query tiles, so every K / V
+// byte is fetched from the caches once per workgroup and round instead of once per wavefront (4x less traffic; with grouped
+// query heads the sharing is across heads, which also holds when every portion is a single decoded token). All threads load
+// the round's 64 tokens with coalesced 16-byte loads — the NEXT round's loads are issued before the current round is
+// computed — K as [token][d], V as [column][token]; the MFMA operands are 16-byte LDS reads. Softmax, masks and the token
+// permutation are those of the kernel above.
+template <int DK, int DVB, int QT>
+__global__ __launch_bounds__(256) void window_attn_mfma_lds_kernel(
+    const bf16_t* __restrict__ q, int64_t q_stride, const bf16_t* __restrict__ qnorm, float eps, const bf16_t* __restrict__ gate,
+    int64_t gate_stride, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+    const int32_t* __restrict__ block_tables, int64_t bt_stride, int block_size, const int32_t* __restrict__ cu_q,
+    const int32_t* __restrict__ ctx0, int nseq, int H, int G, int d, int dv, float scale, int window, int bs_shift, int hw,
+    bf16_t* __restrict__ out) {
+  constexpr int QW = 16 * QT, KP = 32 * DK + 8, VP = 64 + 8, VU = DVB / 2;
+  __shared__ __attribute__((aligned(16))) bf16_t Ks[64][KP];
+  __shared__ __attribute__((aligned(16))) bf16_t Vs[16 * DVB][VP];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, qi = lane & 15, gq = lane >> 4;
+  const int hpg = H / G, chunks = hpg / hw;
+  const int g = blockIdx.y / chunks, h = g * hpg + (blockIdx.y % chunks) * hw + (wave % hw);
+  const int tq = 4 / hw, BQ = tq * QW;             // query tiles and queries of the workgroup
+  int btile = blockIdx.x, s = 0, len = 0;
+  for (; s < nseq; ++s) {
+    len = cu_q[s + 1] - cu_q[s];
+    const int tiles = (len + BQ - 1) / BQ;
+    if (btile < tiles) break;
+    btile -= tiles;
+  }
+  if (s >= nseq) return;                            // the whole workgroup leaves
+  const int c0 = ctx0[s];
+  const int rel0 = btile * BQ + (wave / hw) * QW;   // this wavefront's first query inside the portion (may lie beyond its end)
+  const int p_first = c0 + rel0, p_hi = c0 + rel0 + QW - 1;
+  const int b_first = c0 + btile * BQ;
+  const int b_last = c0 + (btile * BQ + BQ - 1 < len ? btile * BQ + BQ - 1 : len - 1);
+  const int bs_mask = block_size - 1;
+  const int32_t* bt = block_tables + (int64_t)s * bt_stride;
+
+  bf16x8_t qb[QT][DK];
+  bool valid_q[QT];
+  int64_t row[QT];
+  int pos[QT];
+#pragma unroll
+  for (int t = 0; t < QT; ++t) {
+    const int rel = rel0 + t * 16 + qi;
+    valid_q[t] = rel < len;
+    row[t] = (int64_t)cu_q[s] + (valid_q[t] ? rel : len - 1);
+    pos[t] = c0 + rel;
+    float qv[DK][8];
+    float ss = 0.f;
+    const bf16_t* qp = q + row[t] * q_stride + (int64_t)h * d;
+#pragma unroll
+    for (int c = 0; c < DK; ++c)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int col = c * 32 + gq * 8 + e;
+        qv[c][e] = col < d ? (float)qp[col] : 0.f;
+        ss += qv[c][e] * qv[c][e];
+      }
+    float r = scale;
+    if (qnorm) {
+      ss += __shfl_xor(ss, 16, 64);
+      ss += __shfl_xor(ss, 32, 64);
+      r *= rsqrtf(ss / (float)d + eps);
+    }
+#pragma unroll
+    for (int c = 0; c < DK; ++c)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int col = c * 32 + gq * 8 + e;
+        const float w = (qnorm && col < d) ? (float)qnorm[col] : 1.f;
+        qb[t][c][e] = (bf16_t)(qv[c][e] * r * w);
+      }
+  }
+  float m[QT], lsum[QT];
+  f32x4_t oacc[QT][DVB];
+#pragma unroll
+  for (int t = 0; t < QT; ++t) {
+    m[t] = -1e30f;
+    lsum[t] = 0.f;
+#pragma unroll
+    for (int db = 0; db < DVB; ++db) oacc[t][db] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  }
+  const u32x4_t zero4 = u32x4_t{0u, 0u, 0u, 0u};
+  // staging: thread -> DK 16-byte units of K (token, 8 of d) and VU units of V (column, 8 tokens)
+  u32x4_t kf[DK], vf[VU];
+  auto fetch = [&](int j0) {
+#pragma unroll
+    for (int i = 0; i < DK; ++i) {
+      const int u = tid + i * 256, tok = u / (4 * DK), part = u - tok * (4 * DK);
+      const int j = j0 + tok;
+      kf[i] = zero4;
+      if (j <= b_last && part * 8 < d) {
+        const int pg = bs_shift >= 0 ? j >> bs_shift : j / block_size;
+        const int off = bs_shift >= 0 ? j & bs_mask : j - pg * block_size;
+        kf[i] = *(const u32x4_t*)(k_cache + (((int64_t)bt[pg] * block_size + off) * G + g) * d + part * 8);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < VU; ++i) {
+      const int u = tid + i * 256, col = u >> 3, grp = u & 7;
+      const int j = j0 + grp * 8;
+      vf[i] = zero4;
+      if (j <= b_last && col < dv) {
+        const int pg = bs_shift >= 0 ? j >> bs_shift : j / block_size;
+        const int off = bs_shift >= 0 ? j & bs_mask : j - pg * block_size;
+        vf[i] = *(const u32x4_t*)(v_cache + (((int64_t)bt[pg] * G + g) * dv + col) * block_size + off);
+      }
+    }
+  };
+  const int lo = window > 0 ? (b_first - window + 1 > 0 ? b_first - window + 1 : 0) : 0;
+  int j0 = lo & ~31;
+  fetch(j0);
+  for (; j0 <= b_last; j0 += 64) {
+    __syncthreads();                                // the previous round's readers are done
+#pragma unroll
+    for (int i = 0; i < DK; ++i) {
+      const int u = tid + i * 256, tok = u / (4 * DK), part = u - tok * (4 * DK);
+      *(u32x4_t*)&Ks[tok][part * 8] = kf[i];
+    }
+#pragma unroll
+    for (int i = 0; i < VU; ++i) {
+      const int u = tid + i * 256, col = u >> 3, grp = u & 7;
+      *(u32x4_t*)&Vs[col][grp * 8] = vf[i];
+    }
+    __syncthreads();
+    if (j0 + 64 <= b_last) fetch(j0 + 64);
+    // a wavefront whose queries all lie before the round's tokens (or beyond the portion) has nothing to add
+    if (j0 > p_hi || rel0 >= len || (window > 0 && j0 + 63 < p_first - window + 1)) continue;
+    const bool interior = j0 + 63 <= p_first && (window <= 0 || p_hi - j0 < window);
+    f32x4_t sacc[QT][4];
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb) {
+#pragma unroll
+      for (int t = 0; t < QT; ++t) sacc[t][kb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      const int tok = (kb >> 1) * 32 + (qi >> 2) * 8 + (kb & 1) * 4 + (qi & 3);
+#pragma unroll
+      for (int c = 0; c < DK; ++c) {
+        const bf16x8_t a = *(const bf16x8_t*)&Ks[tok][c * 32 + gq * 8];
+#pragma unroll
+        for (int t = 0; t < QT; ++t) sacc[t][kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qb[t][c], sacc[t][kb], 0, 0, 0);
+      }
+    }
+    bf16x8_t pb[QT][2];
+#pragma unroll
+    for (int t = 0; t < QT; ++t) {
+      float mx = m[t];
+      unsigned okbits = 0xffffu;
+      if (!interior) {
+        okbits = 0u;
+#pragma unroll
+        for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int j = j0 + (kb >> 1) * 32 + gq * 8 + (kb & 1) * 4 + r;
+            const bool ok = valid_q[t] && j <= pos[t] && (window <= 0 || pos[t] - j < window);
+            okbits |= ok ? (1u << (kb * 4 + r)) : 0u;
+          }
+      }
+#pragma unroll
+      for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (okbits & (1u << (kb * 4 + r))) mx = fmaxf(mx, sacc[t][kb][r]);
+      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float alpha = __expf(m[t] - mx);
+      m[t] = mx;
+      float ls = lsum[t] * alpha;
+#pragma unroll
+      for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float p = (okbits & (1u << (kb * 4 + r))) ? __expf(sacc[t][kb][r] - mx) : 0.f;
+          ls += p;
+          pb[t][kb >> 1][(kb & 1) * 4 + r] = (bf16_t)p;
+        }
+      lsum[t] = ls;
+      if (__ballot(alpha != 1.f) != 0ull) {
+#pragma unroll
+        for (int db = 0; db < DVB; ++db) oacc[t][db] *= alpha;
+      }
+    }
+#pragma unroll
+    for (int mg = 0; mg < 2; ++mg)
+#pragma unroll
+      for (int db = 0; db < DVB; ++db) {
+        const bf16x8_t a = *(const bf16x8_t*)&Vs[db * 16 + qi][mg * 32 + gq * 8];
+#pragma unroll
+        for (int t = 0; t < QT; ++t) oacc[t][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb[t][mg], oacc[t][db], 0, 0, 0);
+      }
+  }
+#pragma unroll
+  for (int t = 0; t < QT; ++t) {
+    float ls = lsum[t];
+    ls += __shfl_xor(ls, 16, 64);
+    ls += __shfl_xor(ls, 32, 64);
+    if (!valid_q[t]) continue;
+    const float inv = 1.f / ls;
+    bf16_t* op = out + ((int64_t)row[t] * H + h) * dv;
+    const bf16_t* gp = gate ? gate + row[t] * gate_stride + (int64_t)h * dv : nullptr;
+#pragma unroll
+    for (int db = 0; db < DVB; ++db)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int c = db * 16 + gq * 4 + r;
+        if (c < dv) {
+          float o = oacc[t][db][r] * inv;
+          if (gp) o *= 1.f / (1.f + expf(-(float)gp[c]));
+          op[c] = (bf16_t)o;
+        }
+      }
+  }
+}
+
 template <int DK, int DVB, int QT>
 void launch_mfma_qt(const void* q, int64_t q_stride, const void* qnorm, float eps, const void* gate, int64_t gate_stride,
                     const void* k_cache, const void* v_cache, const int32_t* block_tables, int64_t bt_stride, int block_size,
                     const int32_t* cu_q, const int32_t* ctx0, int nseq, int64_t n, int H, int G, int d, int dv, float scale, int window,
                     void* out, hipStream_t stream) {
-  const int64_t tiles = n / (16 * QT) + nseq;       // an upper bound: every portion may end with a partial tile
   int bs_shift = -1;
   for (int b = 0; b < 31; ++b)
     if ((1 << b) == block_size) bs_shift = b;
+  if constexpr (64 * (32 * DK + 8) * 2 + 16 * DVB * 72 * 2 <= 65536) {
+    if (!g_no_lds) {
+      const int hpg = H / G, hw = hpg % 4 == 0 ? 4 : (hpg % 2 == 0 ? 2 : 1);
+      const int bq = (4 / hw) * 16 * QT;
+      const int64_t btiles = n / bq + nseq;         // an upper bound: every portion may end with a partial tile
+      window_attn_mfma_lds_kernel<DK, DVB, QT><<<dim3((unsigned)btiles, (unsigned)(G * (hpg / hw))), dim3(256), 0, stream>>>(
+          (const bf16_t*)q, q_stride, (const bf16_t*)qnorm, eps, (const bf16_t*)gate, gate_stride, (const bf16_t*)k_cache,
+          (const bf16_t*)v_cache, block_tables, bt_stride, block_size, cu_q, ctx0, nseq, H, G, d, dv, scale, window, bs_shift, hw,
+          (bf16_t*)out);
+      return;
+    }
+  }
+  const int64_t tiles = n / (16 * QT) + nseq;       // an upper bound: every portion may end with a partial tile
   window_attn_mfma_kernel<DK, DVB, QT><<<dim3((unsigned)((tiles + 3) / 4), H), dim3(256), 0, stream>>>(
       (const bf16_t*)q, q_stride, (const bf16_t*)qnorm, eps, (const bf16_t*)gate, gate_stride, (const bf16_t*)k_cache,
       (const bf16_t*)v_cache, block_tables, bt_stride, block_size, cu_q, ctx0, nseq, H, G, d, dv, scale, window, bs_shift, (bf16_t*)out);
@@ -364,7 +591,10 @@ void launch_mfma(const void* q, int64_t q_stride, const void* qnorm, float eps, 
 
 static int g_force_scalar = 0;
 /* tests: 1 routes bf16 calls through the scalar kernel as well */
-extern "C" void nvs_window_attn_force_scalar(int on) { g_force_scalar = on; }
+extern "C" void nvs_window_attn_force_scalar(int on) {
+  g_force_scalar = on == 1;
+  g_no_lds = on == 2;
+}
 
 extern "C" int nvs_knorm_kvstore(const void* k, const void* v, int64_t stride, int dtype, const void* knorm, float eps, int G, int d,
                                  int dv, int block_size, const int32_t* slots, int64_t n, void* k_cache, void* v_cache, void* stream) {

@@ -56,6 +56,8 @@ def load_library() -> ctypes.CDLL:
         raise NvsError(f"libnvl_seq.so ABI version {lib.nvs_abi_version()} != binding version {ABI_VERSION}; rebuild")
     if os.environ.get("NVL_ATTN_SCALAR") == "1":      # A/B switch: bf16 windowed attention on the scalar kernel too
         lib.nvs_window_attn_force_scalar(1)
+    elif os.environ.get("NVL_ATTN_NO_LDS") == "1":    # ... or on the matrix cores without the LDS-shared K / V tiles
+        lib.nvs_window_attn_force_scalar(2)
     _lib = lib
     return lib
 

@@ -236,10 +236,12 @@ def _plain_attention(q, k, v, H, G, d, dv, scale, window, qn=None, kn=None, gate
 
 @pytest.mark.parametrize("H,G,d,dv,window,block", [(4, 2, 32, 48, 20, 16), (3, 3, 64, 128, 64, 64), (8, 1, 16, 16, 1, 16),
                                                    (2, 2, 80, 200, 0, 32), (6, 2, 128, 64, 33, 48)])
-@pytest.mark.parametrize("dtype,path", [(torch.float32, "scalar"), (torch.bfloat16, "matrix"), (torch.bfloat16, "scalar")])
+@pytest.mark.parametrize("dtype,path", [(torch.float32, "scalar"), (torch.bfloat16, "matrix"), (torch.bfloat16, "matrix_own_loads"),
+                                        (torch.bfloat16, "scalar")])
 def test_windowed_attention_against_the_plain_loop(H, G, d, dv, window, block, dtype, path):
-    """float32 takes the one-query-per-wavefront kernel; bfloat16 the matrix-core kernel (16 queries per wavefront), or the
-    scalar one when forced — the path head sizes outside the matrix-core kernel's reach take."""
+    """float32 takes the one-query-per-wavefront kernel; bfloat16 the matrix-core kernel with K / V tiles shared through LDS,
+    the one in which every wavefront loads its own operands (tiles too large for LDS) when forced, or the scalar one when
+    forced — the path head sizes outside the matrix-core kernels' reach take."""
     from nano_vllm_amd import ops_seq
     g = torch.Generator().manual_seed(H * d)
     lens = [70, 5, 129]
@@ -248,7 +250,7 @@ def test_windowed_attention_against_the_plain_loop(H, G, d, dv, window, block, d
     q, k, v = rnd(T, H * d), rnd(T, G * d), rnd(T, G * dv)
     qn, kn, gate = (1 + 0.2 * rnd(d)).to(dtype).float(), (1 + 0.2 * rnd(d)).to(dtype).float(), rnd(T, H * dv)
     order = torch.randperm(sum(-(-L // block) for L in lens) + 3, generator=g).tolist()      # scattered pages
-    ops_seq.load_library().nvs_window_attn_force_scalar(int(path == "scalar"))
+    ops_seq.load_library().nvs_window_attn_force_scalar({"scalar": 1, "matrix": 0, "matrix_own_loads": 2}[path])
     try:
         got = _attend(q, k, v, H, G, d, dv, 0.4, window, block, lens, order, qn, kn, gate, dtype=dtype)
     finally:
