@@ -374,6 +374,7 @@ class ModelRunner:
             self.chan.send(_Channel.OP_EXIT)
         self.graphs = {}
         self.graphs_px = {}
+        self.sgraphs = {}
         torch.cuda.synchronize()
         if self.world_size > 1:
             from .. import tp
@@ -873,6 +874,13 @@ class ModelRunner:
                 ("ctx0", np.int32, (ns,)), ("sslot", np.int32, (ns,)), ("temps", np.float32, (ns,)), ("bt", np.int32, (ns, w)),
             ], self.device)
             self.step_count = 0
+            # decode-only steps (every sequence brings one token) replay a hipGraph per batch bucket: model, logits and
+            # sampler, on the static staging block. Rows beyond the batch are padding: one token at position 0 in a scratch
+            # state slot, no K/V store, page 0 to read, greedy — their results are never looked at.
+            self.graph_bs = sorted({b for b in (1, 2, 4, 8) if b <= ns} | set(range(16, ns + 1, 16)) | {ns})
+            self.sgraphs: dict[int, torch.cuda.CUDAGraph] = {}
+            self._sgraph_pool = None
+            self.scratch_slot = cfg.max_num_seqs
             self.tokens_dev = torch.zeros(ns, dtype=torch.int64, device=self.device)
             self.tokens_host = torch.zeros(ns, dtype=torch.int64, device="cpu", pin_memory=True)
             self._allocate_stateful_caches()
@@ -889,7 +897,8 @@ class ModelRunner:
         block_bytes = max(per_token * self.block_size, 1)
         for m in st_layers:                                       # state first: small, and it is not optional
             for name, shape in m.state_shapes().items():
-                setattr(m, name, torch.zeros(cfg.max_num_seqs, *shape, dtype=torch.float32, device=self.device))
+                # (one slot more than sequences: the scratch slot of a captured decode step's padding rows)
+                setattr(m, name, torch.zeros(cfg.max_num_seqs + 1, *shape, dtype=torch.float32, device=self.device))
         if cfg.num_kvcache_blocks <= 0:
             free, total = torch.cuda.mem_get_info()
             # no profiling pass (it would need pages): activations of the largest step are bounded by the widest fused
@@ -907,9 +916,10 @@ class ModelRunner:
             m.v_cache = torch.zeros(slots, *vs, dtype=self.dtype, device=self.device)
             m.block_size = self.block_size
 
-    def prepare_portions(self, seqs: list[Sequence], want: list[list[int]] | None = None) -> dict:
+    def prepare_portions(self, seqs: list[Sequence], want: list[list[int]] | None = None, pad_to: int = 0) -> dict:
         """Fill the staging block for a packed step: sequence i contributes tokens [num_cached_tokens, + num_scheduled_tokens).
-        `want[i]`: indices INSIDE portion i whose logits the caller asks for (default: the portion's last token)."""
+        `want[i]`: indices INSIDE portion i whose logits the caller asks for (default: the portion's last token).
+        `pad_to`: number of portions a captured step expects; the rest are padding rows (see _init_stateful)."""
         st = self.sstage
         ev = st.uploaded[0]
         if ev is not None:
@@ -940,7 +950,53 @@ class ModelRunner:
                 a["rows"][nrows] = n + r
                 nrows += 1
             n += lq
-        return dict(n=n, ns=len(seqs), nrows=nrows)
+        for i in range(len(seqs), pad_to):
+            a["ids"][n] = 0
+            a["pos"][n] = 0
+            a["slots"][n] = -1
+            a["tseq"][n] = i
+            a["cu_q"][i + 1] = n + 1
+            a["ctx0"][i] = 0
+            a["sslot"][i] = self.scratch_slot
+            a["temps"][i] = 0.0
+            a["rkey"][i] = 0
+            a["bt"][i, :] = 0
+            a["rows"][nrows] = n
+            nrows += 1
+            n += 1
+        return dict(n=n, ns=max(len(seqs), pad_to), nrows=nrows)
+
+    def _ensure_sampler(self):
+        if self.sampler is None:
+            ops.load_library()
+            self.sampler = Sampler(seed=self.config.seed, max_rows=self.config.max_num_seqs)
+
+    @torch.inference_mode()
+    def _decode_body(self, bs: int) -> None:
+        """A decode-only step of `bs` rows on the static staging block: model, logits, sampler (captured per bucket)."""
+        from ..ops_seq import Portions
+        t = self.sstage.t
+        por = Portions(t["cu_q"], t["ctx0"], t["sslot"], t["tseq"], bs, bs)
+        set_context(True, slot_mapping=t["slots"][:bs], block_tables=t["bt"][:bs], portions=por)
+        x = self.model(t["ids"][:bs], t["pos"][:bs])
+        logits = self.model.compute_logits(x, t["rows"], bs)
+        self.sampler(logits, t["temps"][:bs], out=self.tokens_dev[:bs], offset_dev=t["rng"][:1], row_keys=t["rkey"][:bs])
+        reset_context()
+
+    @torch.inference_mode()
+    def _capture_decode(self, bs: int) -> None:
+        """Capture bucket `bs` on an all-padding image (the warm-up run must not advance any sequence's state)."""
+        self.prepare_portions([], pad_to=bs)
+        self.sstage.upload()
+        self._decode_body(bs)                                   # warm-up: allocator, GEMM heuristics, sampler workspace
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, self._sgraph_pool):
+            self._decode_body(bs)
+        if self._sgraph_pool is None:
+            self._sgraph_pool = graph.pool()
+        self.sgraphs[bs] = graph
+        torch.cuda.synchronize()
 
     @torch.inference_mode()
     def _launch_portions(self, info: dict) -> torch.Tensor:
@@ -959,15 +1015,23 @@ class ModelRunner:
 
     def run_portions(self, seqs: list[Sequence]) -> list[int]:
         """One packed step, one sampled token per sequence (from its portion's last token)."""
-        info = self.prepare_portions(seqs)
+        self._ensure_sampler()
+        ns = len(seqs)
+        bucket = 0
+        if not self.enforce_eager and all(s.num_scheduled_tokens == 1 for s in seqs):
+            bucket = next(b for b in self.graph_bs if b >= ns)
+            if bucket not in self.sgraphs:
+                self._capture_decode(bucket)
+        info = self.prepare_portions(seqs, pad_to=bucket)
         self._next_rng(self.sstage)
-        logits = self._launch_portions(info)
-        ns, t = info["ns"], self.sstage.t
-        if self.sampler is None:
-            ops.load_library()
-            self.sampler = Sampler(seed=self.config.seed, max_rows=self.config.max_num_seqs)
-        with torch.inference_mode():
-            self.sampler(logits, t["temps"][:ns], out=self.tokens_dev[:ns], offset_dev=t["rng"][:1], row_keys=t["rkey"][:ns])
+        if bucket:
+            self.sstage.upload()
+            self.sgraphs[bucket].replay()
+        else:
+            logits = self._launch_portions(info)
+            t = self.sstage.t
+            with torch.inference_mode():
+                self.sampler(logits, t["temps"][:ns], out=self.tokens_dev[:ns], offset_dev=t["rng"][:1], row_keys=t["rkey"][:ns])
         self.tokens_host[:ns].copy_(self.tokens_dev[:ns], non_blocking=True)
         torch.cuda.current_stream().synchronize()
         return self.tokens_host[:ns].tolist()

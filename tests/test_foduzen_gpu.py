@@ -422,19 +422,23 @@ def test_long_decoding_past_every_window_and_many_pages(checkpoints):
         llm.exit()
 
 
+@pytest.mark.parametrize("eager", [True, False])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_greedy_generation_through_generate_matches_the_plain_model(checkpoints, dtype):
+def test_greedy_generation_through_generate_matches_the_plain_model(checkpoints, dtype, eager):
     """LLM.generate(): the scheduler admits, chunks (a token budget smaller than the longest prompt) and decodes; every
-    generated token must be the plain model's argmax wherever its margin exceeds the serving precision."""
+    generated token must be the plain model's argmax wherever its margin exceeds the serving precision. `eager=False`:
+    decode-only steps replay captured graphs (three batch buckets here, padded rows included), with eager prefill steps
+    between the replays."""
     from nano_vllm_amd import LLM, SamplingParams
     path = checkpoints[0]
     ref = plain.Model.load(path)
     g = torch.Generator().manual_seed(21)
     prompts = [torch.randint(0, ref.cfg["vocab"], (n,), generator=g).tolist() for n in (5, 70, 33, 1, 64, 18)]
     llm = LLM(path, dtype=dtype, kvcache_block_size=16, num_kvcache_blocks=30, max_num_seqs=4, max_num_batched_tokens=48,
-              max_model_len=256, enforce_eager=True)
+              max_model_len=256, enforce_eager=eager)
     try:
         outs = llm.generate(prompts, SamplingParams(temperature=0.0, max_tokens=12, ignore_eos=True), use_tqdm=False)
+        assert eager or llm.model_runner.sgraphs, "decode steps were meant to replay graphs"
         assert llm.scheduler.block_manager.num_free == 30 and llm.scheduler.state_slots.num_free == 4
     finally:
         llm.exit()
