@@ -2,6 +2,7 @@
 // form), gated group norm. State lives in 32-bit in per-sequence slots; a portion whose first token is position 0 starts
 // from zeros whatever the slot holds.
 #include "seq_common.h"
+#include <stdlib.h>
 
 namespace {
 
@@ -104,22 +105,22 @@ __global__ void rglru_scan_kernel(const float* __restrict__ gates, const float* 
 }
 
 // ---- state-space-duality recurrence -------------------------------------------------------------------------------
-// One workgroup per (portion, head), P * NG threads: thread (p, g) = (tid / NG, tid % NG) keeps the 16 state entries
-// S[p][16 g .. 16 g + 15] in registers (state memory is [heads][P][N], n fastest: a thread's entries are contiguous).
+// One workgroup per (portion, head), (P / PP) * NG threads: thread (tid / NG, g = tid % NG) keeps the 16 state entries
+// S[p][16 g .. 16 g + 15] of PP consecutive p in registers (state memory is [heads][P][N], n fastest: a thread's entries are contiguous).
 // Tokens go in rounds of TB: the round's x | B | C | dt | decay are staged in LDS by all threads, then every token costs 16 x (2 FMA + 1 MUL) per thread, LDS
 // reads that vectorise, and log2(NG) shuffles for y[p] = sum_n S C: the NG threads of a p are neighbouring lanes.
 constexpr int SSD_R = 16;      // state entries per thread
-constexpr int SSD_U = 6;       // staging loads a thread keeps in flight
+constexpr int SSD_TB = 16;     // tokens per LDS round
 
-template <typename T>
-__global__ __launch_bounds__(1024) void ssd_scan_kernel(const float* __restrict__ xbc, const T* __restrict__ proj, int64_t proj_stride, int64_t dt_col,
+template <typename T, int PP>     // PP head-size entries per thread: the B / C values read from LDS serve PP state rows
+__global__ __launch_bounds__(PP == 4 ? 256 : 1024) void ssd_scan_kernel(const float* __restrict__ xbc, const T* __restrict__ proj, int64_t proj_stride, int64_t dt_col,
                                 const T* __restrict__ dt_bias, const T* __restrict__ A_log, const T* __restrict__ Dp, int heads,
                                 int P, int N, int G, int NG, int TB, const int32_t* __restrict__ cu_q,
                                 const int32_t* __restrict__ ctx0, const int32_t* __restrict__ slot, float* __restrict__ S,
                                 float* __restrict__ y) {
   extern __shared__ __attribute__((aligned(16))) float lds[];   // [TB][per]: x (P) | B (NP) | C (NP) | dt, NP = 16 NG, zero padded
   const int s = blockIdx.y, h = blockIdx.x, tid = threadIdx.x, nthreads = blockDim.x;
-  const int g = tid & (NG - 1), p = tid / NG;
+  const int g = tid & (NG - 1), p = (tid / NG) * PP;          // this thread's first p
   const int64_t q0 = cu_q[s], q1 = cu_q[s + 1];
   if (q1 <= q0) return;
   const int NP = NG * SSD_R, P4 = (P + 3) & ~3, per = P4 + 2 * NP + 4;    // every part starts 16-byte aligned
@@ -127,75 +128,103 @@ __global__ __launch_bounds__(1024) void ssd_scan_kernel(const float* __restrict_
   const int64_t row = inner + 2 * G * N;
   const float A = -expf(ldf(A_log + h)), Dh = ldf(Dp + h), dtb = ldf(dt_bias + h);
   float* Sh = S + (((int64_t)slot[s] * heads + h) * P + p) * N + g * SSD_R;
-  float st[SSD_R];
+  float st[PP][SSD_R];
   const bool fresh = ctx0[s] == 0;
 #pragma unroll
-  for (int r = 0; r < SSD_R; ++r) st[r] = (!fresh && g * SSD_R + r < N) ? Sh[r] : 0.f;
+  for (int i = 0; i < PP; ++i)
+#pragma unroll
+    for (int r = 0; r < SSD_R; ++r) st[i][r] = (!fresh && g * SSD_R + r < N) ? Sh[(int64_t)i * N + r] : 0.f;
 
   const float* xh = xbc + h * P;
+  float* yh = y + h * P + p;
   const float* Bg = xbc + inner + grp * N;
   const float* Cg = Bg + G * N;
   for (int64_t tb = q0; tb < q1; tb += TB) {
     const int cnt = (int)((q1 - tb) < TB ? (q1 - tb) : TB);
     __syncthreads();                                // the previous round's readers are done
     // stage the round: other workgroups of the CU compute meanwhile (LDS and registers leave room for several)
-    // (SSD_U independent loads per thread are in flight before the first LDS store)
-    const int total = cnt * per;
-    for (int base = tid; base < total; base += SSD_U * nthreads) {
-      float v[SSD_U];
+    // a thread stages ONE column of the image for all tokens of the round: the column is classified once, the 16 loads are
+    // independent and in flight together, and for a fixed token neighbouring threads read neighbouring addresses
+    for (int c = tid; c < per; c += nthreads) {
+      const float* src = nullptr;                   // a 32-bit source with row stride `row`
+      int kind = 0;                                 // 0: padding (zero), 1: x / B / C, 2: step size, 3: decay
+      if (c < P) {
+        src = xh + c, kind = 1;
+      } else if (c >= P4 && c < P4 + NP) {
+        if (c - P4 < N) src = Bg + (c - P4), kind = 1;
+      } else if (c >= P4 + NP && c < P4 + 2 * NP) {
+        if (c - P4 - NP < N) src = Cg + (c - P4 - NP), kind = 1;
+      } else if (c == P4 + 2 * NP) {
+        kind = 2;
+      } else if (c == P4 + 2 * NP + 1) {
+        kind = 3;
+      }
+      float v[SSD_TB];
 #pragma unroll
-      for (int u = 0; u < SSD_U; ++u) {
-        const int idx = base + u * nthreads;
-        v[u] = 0.f;
-        if (idx < total) {
-          const int k = idx / per, c = idx - k * per;
-          const int64_t t = tb + k;
-          if (c < P) {
-            v[u] = xh[t * row + c];
-          } else if (c >= P4 && c < P4 + NP) {
-            if (c - P4 < N) v[u] = Bg[t * row + (c - P4)];
-          } else if (c >= P4 + NP && c < P4 + 2 * NP) {
-            if (c - P4 - NP < N) v[u] = Cg[t * row + (c - P4 - NP)];
-          } else if (c >= P4 + 2 * NP && c <= P4 + 2 * NP + 1) {
-            v[u] = ldf(proj + t * proj_stride + dt_col + h);
-          }
+      for (int k = 0; k < SSD_TB; ++k) {
+        v[k] = 0.f;
+        if (k < cnt) {
+          if (kind == 1) v[k] = src[(tb + k) * row];
+          if (kind >= 2) v[k] = ldf(proj + (tb + k) * proj_stride + dt_col + h);
         }
       }
 #pragma unroll
-      for (int u = 0; u < SSD_U; ++u) {
-        const int idx = base + u * nthreads;
-        if (idx < total) {
-          const int c = idx % per;
-          float w = v[u];
-          if (c >= P4 + 2 * NP && c <= P4 + 2 * NP + 1) {          // step size, and the decay it gives
+      for (int k = 0; k < SSD_TB; ++k) {
+        if (k < cnt) {
+          float w = v[k];
+          if (kind >= 2) {
             w = softplusf_(w + dtb);
-            if (c == P4 + 2 * NP + 1) w = expf(A * w);
+            if (kind == 3) w = expf(A * w);
           }
-          lds[idx] = w;
+          lds[k * per + c] = w;
         }
       }
     }
     __syncthreads();
-    for (int k = 0; k < cnt; ++k) {
+    // one token: S <- dA S + dt B x, y = S . C (+ D x). Tokens of a full round are unrolled four at a time so that the LDS
+    // reads and the shuffle chains of neighbouring tokens overlap (only the 16 state FMAs of a token wait for the one before)
+    auto token = [&](int k) {
       const float* tp = lds + k * per;
       const float dt = tp[P4 + 2 * NP], dA = tp[P4 + 2 * NP + 1];
-      const float xv = tp[p];
       const float* Bp = (const float*)__builtin_assume_aligned(tp + P4 + g * SSD_R, 16);
       const float* Cp = (const float*)__builtin_assume_aligned(Bp + NP, 16);
-      const float dx = dt * xv;
-      float acc = 0.f;
+      float bv[SSD_R], cv[SSD_R];
 #pragma unroll
-      for (int r = 0; r < SSD_R; ++r) {
-        st[r] = dA * st[r] + Bp[r] * dx;
-        acc += st[r] * Cp[r];
+      for (int r = 0; r < SSD_R; ++r) bv[r] = Bp[r], cv[r] = Cp[r];
+      float out[PP];
+#pragma unroll
+      for (int i = 0; i < PP; ++i) {
+        const float xv = tp[p + i];
+        const float dx = dt * xv;
+        float acc0 = 0.f, acc1 = 0.f;
+#pragma unroll
+        for (int r = 0; r < SSD_R; r += 2) {
+          st[i][r] = dA * st[i][r] + bv[r] * dx;
+          st[i][r + 1] = dA * st[i][r + 1] + bv[r + 1] * dx;
+          acc0 += st[i][r] * cv[r];
+          acc1 += st[i][r + 1] * cv[r + 1];
+        }
+        float acc = acc0 + acc1;
+        for (int o = NG >> 1; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
+        out[i] = acc + Dh * xv;
       }
-      for (int o = NG >> 1; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
-      if (g == 0) y[(tb + k) * inner + h * P + p] = acc + Dh * xv;
+      if (g == 0) {
+#pragma unroll
+        for (int i = 0; i < PP; ++i) yh[(tb + k) * inner + i] = out[i];
+      }
+    };
+    if (cnt == SSD_TB) {
+#pragma unroll 4
+      for (int k = 0; k < 16; ++k) token(k);
+    } else {
+      for (int k = 0; k < cnt; ++k) token(k);
     }
   }
 #pragma unroll
-  for (int r = 0; r < SSD_R; ++r)
-    if (g * SSD_R + r < N) Sh[r] = st[r];
+  for (int i = 0; i < PP; ++i)
+#pragma unroll
+    for (int r = 0; r < SSD_R; ++r)
+      if (g * SSD_R + r < N) Sh[(int64_t)i * N + r] = st[i][r];
 }
 
 // ---- gate, then group RMS norm ------------------------------------------------------------------------------------
@@ -269,13 +298,25 @@ extern "C" int nvs_ssd_scan(const float* xbc, const void* proj, int64_t proj_str
   if (n == 0 || nseq == 0) return NVS_OK;
   int ng = 1;
   while (ng * SSD_R < N) ng <<= 1;                  // a power of two: the threads of one p reduce by lane shuffles
-  NVS_REQUIRE(ng <= 64 && (int64_t)P * ng <= 1024, "nvs_ssd_scan: state %d x head size %d exceeds one workgroup's registers", N, P);
-  const int threads = P * ng, per = ((P + 3) & ~3) + 2 * ng * SSD_R + 4;
-  const int tb = 16;                                // tokens per LDS round
+  int ng0 = 1;
+  while (ng0 * SSD_R < N) ng0 <<= 1;
+  // Four rows per thread (PP = 4: a quarter of the LDS reads per FMA) measured SLOWER on the MI355X (4.9 ms against 4.2 ms
+  // for 8 x 2048 tokens, 64 heads of 64 x 128): the scan is bound by the latency of the token chain, which fewer, fatter
+  // wavefronts hide less well, not by LDS bandwidth. NVS_SSD_PP4=1 selects it for measurements.
+  static const bool want4 = getenv("NVS_SSD_PP4") && getenv("NVS_SSD_PP4")[0] == '1';
+  const int pp = (want4 && P % 4 == 0 && (P / 4) * ng0 <= 256) ? 4 : 1;
+  NVS_REQUIRE(ng <= 64 && (int64_t)(P / pp) * ng <= 1024, "nvs_ssd_scan: state %d x head size %d exceeds one workgroup's registers", N, P);
+  const int threads = (P / pp) * ng, per = ((P + 3) & ~3) + 2 * ng * SSD_R + 4;
+  const int tb = SSD_TB;                            // tokens per LDS round
   const size_t lds = (size_t)tb * per * sizeof(float);
-  NVS_DISPATCH(dtype, ssd_scan_kernel<T><<<dim3(heads, (unsigned)nseq), dim3(threads), lds, (hipStream_t)stream>>>(
-                          xbc, (const T*)proj, proj_stride, dt_col, (const T*)dt_bias, (const T*)A_log, (const T*)D, heads, P, N, G, ng, tb,
-                          cu_q, ctx0, slot, S, y));
+  if (pp == 4)
+    NVS_DISPATCH(dtype, ssd_scan_kernel<T, 4><<<dim3(heads, (unsigned)nseq), dim3(threads), lds, (hipStream_t)stream>>>(
+                            xbc, (const T*)proj, proj_stride, dt_col, (const T*)dt_bias, (const T*)A_log, (const T*)D, heads, P, N, G, ng,
+                            tb, cu_q, ctx0, slot, S, y));
+  else
+    NVS_DISPATCH(dtype, ssd_scan_kernel<T, 1><<<dim3(heads, (unsigned)nseq), dim3(threads), lds, (hipStream_t)stream>>>(
+                            xbc, (const T*)proj, proj_stride, dt_col, (const T*)dt_bias, (const T*)A_log, (const T*)D, heads, P, N, G, ng,
+                            tb, cu_q, ctx0, slot, S, y));
   return nvs_check_launch("nvs_ssd_scan");
 }
 
