@@ -111,9 +111,10 @@ __global__ void rglru_scan_kernel(const float* __restrict__ gates, const float* 
 // reads that vectorise, and log2(NG) shuffles for y[p] = sum_n S C: the NG threads of a p are neighbouring lanes.
 constexpr int SSD_R = 16;      // state entries per thread
 constexpr int SSD_TB = 16;     // tokens per LDS round
+constexpr int SSD_SB = 8;      // tokens whose cross-lane sums are taken together
 
 template <typename T, int PP>     // PP head-size entries per thread: the B / C values read from LDS serve PP state rows
-__global__ __launch_bounds__(PP == 4 ? 256 : 1024) void ssd_scan_kernel(const float* __restrict__ xbc, const T* __restrict__ proj, int64_t proj_stride, int64_t dt_col,
+__global__ __launch_bounds__(PP == 4 ? 256 : (PP == 2 ? 512 : 1024)) void ssd_scan_kernel(const float* __restrict__ xbc, const T* __restrict__ proj, int64_t proj_stride, int64_t dt_col,
                                 const T* __restrict__ dt_bias, const T* __restrict__ A_log, const T* __restrict__ Dp, int heads,
                                 int P, int N, int G, int NG, int TB, const int32_t* __restrict__ cu_q,
                                 const int32_t* __restrict__ ctx0, const int32_t* __restrict__ slot, float* __restrict__ S,
@@ -181,9 +182,8 @@ __global__ __launch_bounds__(PP == 4 ? 256 : 1024) void ssd_scan_kernel(const fl
       }
     }
     __syncthreads();
-    // one token: S <- dA S + dt B x, y = S . C (+ D x). Tokens of a full round are unrolled four at a time so that the LDS
-    // reads and the shuffle chains of neighbouring tokens overlap (only the 16 state FMAs of a token wait for the one before)
-    auto token = [&](int k) {
+    // one token: S <- dA S + dt B x; returns this thread's share of y = S . C for each of its rows
+    auto token = [&](int k, float (&part)[PP], float (&xs)[PP]) {
       const float* tp = lds + k * per;
       const float dt = tp[P4 + 2 * NP], dA = tp[P4 + 2 * NP + 1];
       const float* Bp = (const float*)__builtin_assume_aligned(tp + P4 + g * SSD_R, 16);
@@ -191,7 +191,6 @@ __global__ __launch_bounds__(PP == 4 ? 256 : 1024) void ssd_scan_kernel(const fl
       float bv[SSD_R], cv[SSD_R];
 #pragma unroll
       for (int r = 0; r < SSD_R; ++r) bv[r] = Bp[r], cv[r] = Cp[r];
-      float out[PP];
 #pragma unroll
       for (int i = 0; i < PP; ++i) {
         const float xv = tp[p + i];
@@ -204,20 +203,45 @@ __global__ __launch_bounds__(PP == 4 ? 256 : 1024) void ssd_scan_kernel(const fl
           acc0 += st[i][r] * cv[r];
           acc1 += st[i][r + 1] * cv[r + 1];
         }
-        float acc = acc0 + acc1;
-        for (int o = NG >> 1; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
-        out[i] = acc + Dh * xv;
-      }
-      if (g == 0) {
-#pragma unroll
-        for (int i = 0; i < PP; ++i) yh[(tb + k) * inner + i] = out[i];
+        part[i] = acc0 + acc1;
+        xs[i] = xv;
       }
     };
     if (cnt == SSD_TB) {
-#pragma unroll 4
-      for (int k = 0; k < 16; ++k) token(k);
+      // a full round: the cross-lane sums of all its tokens are taken together AFTER the token loop — a shuffle per token
+      // would put a wait for every outstanding LDS access into each step of the recurrence
+#pragma unroll 1
+      for (int k0 = 0; k0 < SSD_TB; k0 += SSD_SB) {
+        float part[SSD_SB][PP], xs[SSD_SB][PP];
+#pragma unroll
+        for (int k = 0; k < SSD_SB; ++k) token(k0 + k, part[k], xs[k]);
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+          if (o < NG) {
+#pragma unroll
+            for (int k = 0; k < SSD_SB; ++k)
+#pragma unroll
+              for (int i = 0; i < PP; ++i) part[k][i] += __shfl_xor(part[k][i], o, 64);
+          }
+        }
+        if (g == 0) {
+#pragma unroll
+          for (int k = 0; k < SSD_SB; ++k)
+#pragma unroll
+            for (int i = 0; i < PP; ++i) yh[(tb + k0 + k) * inner + i] = part[k][i] + Dh * xs[k][i];
+        }
+      }
     } else {
-      for (int k = 0; k < cnt; ++k) token(k);
+      for (int k = 0; k < cnt; ++k) {
+        float part[PP], xs[PP];
+        token(k, part, xs);
+#pragma unroll
+        for (int i = 0; i < PP; ++i) {
+          float acc = part[i];
+          for (int o = NG >> 1; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
+          if (g == 0) yh[(tb + k) * inner + i] = acc + Dh * xs[i];
+        }
+      }
     }
   }
 #pragma unroll
@@ -300,16 +324,22 @@ extern "C" int nvs_ssd_scan(const float* xbc, const void* proj, int64_t proj_str
   while (ng * SSD_R < N) ng <<= 1;                  // a power of two: the threads of one p reduce by lane shuffles
   int ng0 = 1;
   while (ng0 * SSD_R < N) ng0 <<= 1;
-  // Four rows per thread (PP = 4: a quarter of the LDS reads per FMA) measured SLOWER on the MI355X (4.9 ms against 4.2 ms
-  // for 8 x 2048 tokens, 64 heads of 64 x 128): the scan is bound by the latency of the token chain, which fewer, fatter
-  // wavefronts hide less well, not by LDS bandwidth. NVS_SSD_PP4=1 selects it for measurements.
-  static const bool want4 = getenv("NVS_SSD_PP4") && getenv("NVS_SSD_PP4")[0] == '1';
-  const int pp = (want4 && P % 4 == 0 && (P / 4) * ng0 <= 256) ? 4 : 1;
+  // Rows per thread: the 32 B / C values a thread reads from LDS per token serve PP rows, and the scan is bound by the LDS
+  // pipe at PP = 1 (counters: 21 LDS instructions against 93 VALU per wavefront and token, 8 of them 16-byte reads). PP = 4
+  // leaves one wavefront per SIMD and is latency-bound instead (measured slower); PP = 2 is the default where it fits.
+  // NVS_SSD_PP = 1 / 2 / 4 overrides for measurements.
+  static const int forced = getenv("NVS_SSD_PP") ? atoi(getenv("NVS_SSD_PP")) : 0;
+  int pp = forced ? forced : 2;
+  while (pp > 1 && (P % pp != 0 || (P / pp) * ng0 > (pp == 4 ? 256 : 512))) pp >>= 1;
   NVS_REQUIRE(ng <= 64 && (int64_t)(P / pp) * ng <= 1024, "nvs_ssd_scan: state %d x head size %d exceeds one workgroup's registers", N, P);
   const int threads = (P / pp) * ng, per = ((P + 3) & ~3) + 2 * ng * SSD_R + 4;
   const int tb = SSD_TB;                            // tokens per LDS round
   const size_t lds = (size_t)tb * per * sizeof(float);
-  if (pp == 4)
+  if (pp == 2)
+    NVS_DISPATCH(dtype, ssd_scan_kernel<T, 2><<<dim3(heads, (unsigned)nseq), dim3(threads), lds, (hipStream_t)stream>>>(
+                            xbc, (const T*)proj, proj_stride, dt_col, (const T*)dt_bias, (const T*)A_log, (const T*)D, heads, P, N, G, ng,
+                            tb, cu_q, ctx0, slot, S, y));
+  else if (pp == 4)
     NVS_DISPATCH(dtype, ssd_scan_kernel<T, 4><<<dim3(heads, (unsigned)nseq), dim3(threads), lds, (hipStream_t)stream>>>(
                             xbc, (const T*)proj, proj_stride, dt_col, (const T*)dt_bias, (const T*)A_log, (const T*)D, heads, P, N, G, ng,
                             tb, cu_q, ctx0, slot, S, y));
