@@ -418,6 +418,17 @@ __global__ __launch_bounds__(256) void window_attn_mfma_lds_kernel(
   const u32x4_t zero4 = u32x4_t{0u, 0u, 0u, 0u};
   // staging: thread -> DK 16-byte units of K (token, 8 of d) and VU units of V (column, 8 tokens)
   u32x4_t kf[DK], vf[VU];
+  // page ids are looked up one round ahead of the loads that use them: a round's loads then depend on nothing in flight
+  int pgk[DK], pgv;
+  auto lookup = [&](int j0) {
+#pragma unroll
+    for (int i = 0; i < DK; ++i) {
+      const int j = j0 + (tid + i * 256) / (4 * DK);
+      pgk[i] = j <= b_last ? bt[bs_shift >= 0 ? j >> bs_shift : j / block_size] : 0;
+    }
+    const int j = j0 + (tid & 7) * 8;
+    pgv = j <= b_last ? bt[bs_shift >= 0 ? j >> bs_shift : j / block_size] : 0;
+  };
   auto fetch = [&](int j0) {
 #pragma unroll
     for (int i = 0; i < DK; ++i) {
@@ -425,9 +436,8 @@ __global__ __launch_bounds__(256) void window_attn_mfma_lds_kernel(
       const int j = j0 + tok;
       kf[i] = zero4;
       if (j <= b_last && part * 8 < d) {
-        const int pg = bs_shift >= 0 ? j >> bs_shift : j / block_size;
-        const int off = bs_shift >= 0 ? j & bs_mask : j - pg * block_size;
-        kf[i] = *(const u32x4_t*)(k_cache + (((int64_t)bt[pg] * block_size + off) * G + g) * d + part * 8);
+        const int off = bs_shift >= 0 ? j & bs_mask : j % block_size;
+        kf[i] = *(const u32x4_t*)(k_cache + (((int64_t)pgk[i] * block_size + off) * G + g) * d + part * 8);
       }
     }
 #pragma unroll
@@ -436,15 +446,16 @@ __global__ __launch_bounds__(256) void window_attn_mfma_lds_kernel(
       const int j = j0 + grp * 8;
       vf[i] = zero4;
       if (j <= b_last && col < dv) {
-        const int pg = bs_shift >= 0 ? j >> bs_shift : j / block_size;
-        const int off = bs_shift >= 0 ? j & bs_mask : j - pg * block_size;
-        vf[i] = *(const u32x4_t*)(v_cache + (((int64_t)bt[pg] * G + g) * dv + col) * block_size + off);
+        const int off = bs_shift >= 0 ? j & bs_mask : j % block_size;
+        vf[i] = *(const u32x4_t*)(v_cache + (((int64_t)pgv * G + g) * dv + col) * block_size + off);
       }
     }
   };
   const int lo = window > 0 ? (b_first - window + 1 > 0 ? b_first - window + 1 : 0) : 0;
   int j0 = lo & ~31;
+  lookup(j0);
   fetch(j0);
+  lookup(j0 + 64);
   for (; j0 <= b_last; j0 += 64) {
     __syncthreads();                                // the previous round's readers are done
 #pragma unroll
@@ -458,7 +469,10 @@ __global__ __launch_bounds__(256) void window_attn_mfma_lds_kernel(
       *(u32x4_t*)&Vs[col][grp * 8] = vf[i];
     }
     __syncthreads();
-    if (j0 + 64 <= b_last) fetch(j0 + 64);
+    if (j0 + 64 <= b_last) {
+      fetch(j0 + 64);
+      lookup(j0 + 128);
+    }
     // a wavefront whose queries all lie before the round's tokens (or beyond the portion) has nothing to add
     if (j0 > p_hi || rel0 >= len || (window > 0 && j0 + 63 < p_first - window + 1)) continue;
     const bool interior = j0 + 63 <= p_first && (window <= 0 || p_hi - j0 < window);

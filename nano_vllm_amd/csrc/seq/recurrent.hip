@@ -131,10 +131,21 @@ __global__ __launch_bounds__(PP == 4 ? 256 : (PP == 2 ? 512 : 1024)) void ssd_sc
   float* Sh = S + (((int64_t)slot[s] * heads + h) * P + p) * N + g * SSD_R;
   float st[PP][SSD_R];
   const bool fresh = ctx0[s] == 0;
+  const bool vec = (N & 3) == 0;                    // a thread's 16 entries are then four aligned 16-byte pieces
 #pragma unroll
-  for (int i = 0; i < PP; ++i)
+  for (int i = 0; i < PP; ++i) {
+    if (vec) {
 #pragma unroll
-    for (int r = 0; r < SSD_R; ++r) st[i][r] = (!fresh && g * SSD_R + r < N) ? Sh[(int64_t)i * N + r] : 0.f;
+      for (int r = 0; r < SSD_R; r += 4) {
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (!fresh && g * SSD_R + r < N) v = *(const float4*)(Sh + (int64_t)i * N + r);
+        st[i][r] = v.x, st[i][r + 1] = v.y, st[i][r + 2] = v.z, st[i][r + 3] = v.w;
+      }
+    } else {
+#pragma unroll
+      for (int r = 0; r < SSD_R; ++r) st[i][r] = (!fresh && g * SSD_R + r < N) ? Sh[(int64_t)i * N + r] : 0.f;
+    }
+  }
 
   const float* xh = xbc + h * P;
   float* yh = y + h * P + p;
@@ -245,10 +256,17 @@ __global__ __launch_bounds__(PP == 4 ? 256 : (PP == 2 ? 512 : 1024)) void ssd_sc
     }
   }
 #pragma unroll
-  for (int i = 0; i < PP; ++i)
+  for (int i = 0; i < PP; ++i) {
+    if (vec) {
 #pragma unroll
-    for (int r = 0; r < SSD_R; ++r)
-      if (g * SSD_R + r < N) Sh[(int64_t)i * N + r] = st[i][r];
+      for (int r = 0; r < SSD_R; r += 4)
+        if (g * SSD_R + r < N) *(float4*)(Sh + (int64_t)i * N + r) = make_float4(st[i][r], st[i][r + 1], st[i][r + 2], st[i][r + 3]);
+    } else {
+#pragma unroll
+      for (int r = 0; r < SSD_R; ++r)
+        if (g * SSD_R + r < N) Sh[(int64_t)i * N + r] = st[i][r];
+    }
+  }
 }
 
 // ---- gate, then group RMS norm ------------------------------------------------------------------------------------
