@@ -38,7 +38,8 @@ def gelu_tanh(z):
 
 
 def xielu(z, p, q):
-    """z > 0: softplus(p) z^2 + z/2; z <= 0: (1/2 + softplus(q)) (exp(z) - 1 - z) + z/2."""
+    """Quadratic above zero, saturating below, linear coefficient 1/2 on both sides:
+    a = softplus(p), b = 1/2 + softplus(q);  f(z) = a z^2 + z/2 (z > 0),  b (e^z - 1 - z) + z/2 (z <= 0)."""
     ap, aq = softplus(p), 0.5 + softplus(q)
     zn = torch.clamp(z, max=0.0)
     return torch.where(z > 0, ap * z * z + 0.5 * z, aq * (torch.exp(zn) - 1.0 - zn) + 0.5 * z)
