@@ -28,6 +28,10 @@ driver's fields it carries
   parity       : the engine's own T = 0.6 tokens on that sample, judged exactly against the oracle's
                  race keys with the draws replayed (a by-product of the cpu_baseline leg: the timed
                  oracle pass is teacher-forced with the engine's tokens).
+
+`python bench.py --compare-families [--families foduzen,qwen3] [--sizes 1k,4k]` is a different measurement with a line of
+its own (metric "family_compare"): prefill and decode throughput of the Foduzen family at layer sizes of real models beside
+Qwen3 at equal width and depth. The default command above is unchanged by it.
 """
 from __future__ import annotations
 
