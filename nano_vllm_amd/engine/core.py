@@ -256,7 +256,9 @@ class LLMEngine:
         portions, want = [], []
         for e in entries:
             toks = [int(t) for t in e["tokens"]]
-            assert toks, "an entry brings at least one token"
+            if not toks:                        # nothing for this request in this step
+                assert not e.get("want"), "logits were asked of an entry without tokens"
+                continue
             seq = self._replay.get(e["id"])
             if seq is None:
                 seq = self._replay[e["id"]] = self._new_sequence(toks, SamplingParams(temperature=0.0, max_tokens=1))
@@ -268,9 +270,13 @@ class LLMEngine:
             portions.append((seq, len(toks)))
             want.append([int(w) for w in e.get("want", ())])
         assert sum(c for _, c in portions) <= self.config.max_num_batched_tokens, "step exceeds max_num_batched_tokens"
-        batch = self.scheduler.schedule_portions(portions)
-        logits = self.model_runner.call("run_logits", batch, want)
-        self.scheduler.finish_portions(batch)
+        if portions:
+            batch = self.scheduler.schedule_portions(portions)
+            logits = self.model_runner.call("run_logits", batch, want)
+            self.scheduler.finish_portions(batch)
+        else:                                   # a step that brings nothing (it may still end requests)
+            import numpy as np
+            logits = np.zeros((0, self.config.hf_config.vocab_size), dtype=np.float32)
         for name in end:
             seq = self._replay.pop(name, None)
             if seq is not None:

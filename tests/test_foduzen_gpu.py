@@ -473,3 +473,49 @@ def test_sampled_generation_is_reproducible_and_preemption_recomputes_state(chec
         finally:
             llm.exit()
     assert outs[0] == outs[1]
+
+
+def test_the_schedule_replayer_as_a_program(checkpoints, tmp_path):
+    """bin/trace_run as a user starts it: JSON lines in, `done <step>` lines and little-endian float32 files out, pages of
+    64 tokens and four state slots reused as requests end, exit code 0 at the end of its input."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    path = checkpoints[0]
+    ref = plain.Model.load(path)
+    V = ref.cfg["vocab"]
+    g = torch.Generator().manual_seed(31)
+    toks = {k: torch.randint(0, V, (n,), generator=g).tolist() for k, n in (("a", 130), ("b", 70), ("c", 9), ("d", 64), ("e", 100))}
+    want = {k: ref.run(v).numpy() for k, v in toks.items()}
+    steps = [[("a", 100, [0, 99]), ("b", 2, [1])], [("a", 1, [0]), ("b", 60, [3, 59]), ("c", 9, [8])], [("b", 8, [7]), ("a", 29, [28]), ("d", 64, [63])],
+             [("e", 64, [0, 63])], [], [("e", 2, [0, 1])], [("e", 34, [33])]]
+    out = tmp_path / "out"
+    p = subprocess.Popen([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", path, "--dtype", "float32", "--out", str(out),
+                          "--max-tokens", "384"], stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True, cwd=root)
+    at = {k: 0 for k in toks}
+    scale = float(want["a"].std())
+    for n, step in enumerate(steps):
+        entries, rows, end = [], [], []
+        for k, c, w in step:
+            entries.append({"id": k, "tokens": toks[k][at[k]:at[k] + c], "want": w})
+            rows += [(k, at[k] + i) for i in w]
+            at[k] += c
+            if at[k] == len(toks[k]):
+                end.append(k)
+        p.stdin.write(json.dumps({"step": n, "entries": entries, "end": end}) + "\n")
+        p.stdin.flush()
+        while True:
+            line = p.stdout.readline()
+            assert line, "the program ended early"
+            if line.strip() == f"done {n}":
+                break
+        f = out / f"{n}.f32"
+        if rows:
+            got = np.fromfile(f, dtype="<f4").reshape(len(rows), V)
+            exp = np.stack([want[k][i] for k, i in rows])
+            assert rel(got, exp, scale) <= 5e-5, n
+        else:
+            assert not f.exists()
+    p.stdin.close()
+    assert p.wait(timeout=60) == 0
+    assert at == {k: len(v) for k, v in toks.items()}
