@@ -68,10 +68,15 @@ int nvs_rglru_scan(const float* gates, const float* u, const void* ypre, int64_t
 /* State-space-duality recurrence, recurrent form. xbc [n, inner + 2*G*N] 32-bit (x | B | C after convolution + SiLU),
  * dt: column dt_col .. dt_col + heads of proj [n, proj_stride] (`dtype`); dt_bias, A_log, D [heads] (`dtype`). Per head h
  * (group h / (heads / G)), token by token: dt = softplus(dt + dt_bias), S = exp(-exp(A_log) dt) S + dt B x^T,
- * y = S^T C + D x. State memory is [nslots, heads, P, N] (n fastest), 32-bit, advanced. y [n, heads * P] 32-bit. */
+ * y = S^T C + D x. State memory is [nslots, heads, P, N] (n fastest), 32-bit, advanced. y [n, heads * P] 32-bit.
+ * A workgroup walks a (portion, head)'s tokens one after the other; when such pairs are few and portions long (max_q = the
+ * longest portion of the step), portions are cut into segments that are scanned twice — local states from zero, then from
+ * the combined states of the segments before — in `ws` (nvs_ssd_scan_workspace floats; NULL or 0: never segmented). */
+int64_t nvs_ssd_scan_workspace(int heads, int P, int N, int nseq, int64_t max_q);
 int nvs_ssd_scan(const float* xbc, const void* proj, int64_t proj_stride, int64_t dt_col, int dtype, const void* dt_bias,
                  const void* A_log, const void* D, int heads, int P, int N, int G, const int32_t* cu_q, const int32_t* ctx0,
-                 const int32_t* slot, int nseq, int64_t n, float* S, float* y, void* stream);
+                 const int32_t* slot, int nseq, int64_t n, int64_t max_q, float* S, float* y, float* ws, int64_t ws_floats,
+                 void* stream);
 
 /* out = group_rms(y * silu(z)) * w: the gate first, then each of `groups` equal parts of a row by its own root mean square.
  * y [n, inner] 32-bit; z [n, inner] with row stride z_stride (`dtype`); w [inner]; out [n, inner] `dtype`. */

@@ -20,7 +20,7 @@ int nvs_check_launch(const char* what) {
   }
   return NVS_OK;
 }
-extern "C" int nvs_abi_version(void) { return 1; }
+extern "C" int nvs_abi_version(void) { return 2; }   // 2: segmented SSD scan (workspace, longest portion)
 extern "C" const char* nvs_last_error(void) { return g_err; }
 
 namespace {

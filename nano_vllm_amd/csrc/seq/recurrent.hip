@@ -118,12 +118,24 @@ __global__ __launch_bounds__(PP == 4 ? 256 : (PP == 2 ? 512 : 1024)) void ssd_sc
                                 const T* __restrict__ dt_bias, const T* __restrict__ A_log, const T* __restrict__ Dp, int heads,
                                 int P, int N, int G, int NG, int TB, const int32_t* __restrict__ cu_q,
                                 const int32_t* __restrict__ ctx0, const int32_t* __restrict__ slot, float* __restrict__ S,
-                                float* __restrict__ y) {
+                                float* __restrict__ y, int mode, int seg_len, int nseg, float* __restrict__ ws) {
+  // mode 0: the whole portion in one workgroup. Long portions with few (portion, head) pairs are cut into segments of
+  // seg_len tokens (blockIdx.z) and scanned twice, because one workgroup walks its tokens one after the other:
+  //   mode 1: every segment but a portion's last from a ZERO state -> its final state L_k and decay product d_k to `ws`
+  //           (entry 0 of a (portion, head) holds the state the portion starts from);
+  //   mode 2: segment k starts from S_k = d_(k-1) S_(k-1) + L_(k-1), S_0 = entry 0, and produces y; the last one writes the slot.
   extern __shared__ __attribute__((aligned(16))) float lds[];   // [TB][per]: x (P) | B (NP) | C (NP) | dt, NP = 16 NG, zero padded
   const int s = blockIdx.y, h = blockIdx.x, tid = threadIdx.x, nthreads = blockDim.x;
   const int g = tid & (NG - 1), p = (tid / NG) * PP;          // this thread's first p
-  const int64_t q0 = cu_q[s], q1 = cu_q[s + 1];
+  const int64_t p0 = cu_q[s], p1 = cu_q[s + 1];
+  const int seg = blockIdx.z;
+  const int64_t q0 = mode == 0 ? p0 : p0 + (int64_t)seg * seg_len;
+  const int64_t q1 = mode == 0 ? p1 : (q0 + seg_len < p1 ? q0 + seg_len : p1);
   if (q1 <= q0) return;
+  const bool last = q1 == p1;
+  if (mode == 1 && last && seg > 0) return;         // nobody starts from the last segment's state
+  float* wst = ws + ((int64_t)(s * heads + h) * (nseg + 1)) * P * N + (int64_t)p * N + g * SSD_R;   // entry e: + e P N
+  float* wdec = ws + (int64_t)gridDim.y * heads * (nseg + 1) * P * N + (int64_t)(s * heads + h) * (nseg + 1);
   const int NP = NG * SSD_R, P4 = (P + 3) & ~3, per = P4 + 2 * NP + 4;    // every part starts 16-byte aligned
   const int inner = heads * P, grp = h / (heads / G);
   const int64_t row = inner + 2 * G * N;
@@ -132,20 +144,54 @@ __global__ __launch_bounds__(PP == 4 ? 256 : (PP == 2 ? 512 : 1024)) void ssd_sc
   float st[PP][SSD_R];
   const bool fresh = ctx0[s] == 0;
   const bool vec = (N & 3) == 0;                    // a thread's 16 entries are then four aligned 16-byte pieces
-#pragma unroll
-  for (int i = 0; i < PP; ++i) {
+  auto load16 = [&](const float* src, float (&dst)[SSD_R]) {
     if (vec) {
 #pragma unroll
       for (int r = 0; r < SSD_R; r += 4) {
         float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (!fresh && g * SSD_R + r < N) v = *(const float4*)(Sh + (int64_t)i * N + r);
-        st[i][r] = v.x, st[i][r + 1] = v.y, st[i][r + 2] = v.z, st[i][r + 3] = v.w;
+        if (g * SSD_R + r < N) v = *(const float4*)(src + r);
+        dst[r] = v.x, dst[r + 1] = v.y, dst[r + 2] = v.z, dst[r + 3] = v.w;
       }
     } else {
 #pragma unroll
-      for (int r = 0; r < SSD_R; ++r) st[i][r] = (!fresh && g * SSD_R + r < N) ? Sh[(int64_t)i * N + r] : 0.f;
+      for (int r = 0; r < SSD_R; ++r) dst[r] = g * SSD_R + r < N ? src[r] : 0.f;
+    }
+  };
+  auto store16 = [&](float* dst, const float (&src)[SSD_R]) {
+    if (vec) {
+#pragma unroll
+      for (int r = 0; r < SSD_R; r += 4)
+        if (g * SSD_R + r < N) *(float4*)(dst + r) = make_float4(src[r], src[r + 1], src[r + 2], src[r + 3]);
+    } else {
+#pragma unroll
+      for (int r = 0; r < SSD_R; ++r)
+        if (g * SSD_R + r < N) dst[r] = src[r];
+    }
+  };
+#pragma unroll
+  for (int i = 0; i < PP; ++i) {
+#pragma unroll
+    for (int r = 0; r < SSD_R; ++r) st[i][r] = 0.f;
+    if (mode == 2) {
+      load16(wst + (int64_t)i * N, st[i]);          // S_0, then the segments before this one
+      for (int k = 0; k < seg; ++k) {
+        float lk[SSD_R];
+        load16(wst + (int64_t)(k + 1) * P * N + (int64_t)i * N, lk);
+        const float dk = wdec[k + 1];
+#pragma unroll
+        for (int r = 0; r < SSD_R; ++r) st[i][r] = dk * st[i][r] + lk[r];
+      }
+    } else if (!fresh && (mode == 0 || seg == 0)) {
+      load16(Sh + (int64_t)i * N, st[i]);
+    }
+    if (mode == 1 && seg == 0) {                    // the portion's starting state, for mode 2
+      store16(wst + (int64_t)i * N, st[i]);
+#pragma unroll
+      for (int r = 0; r < SSD_R; ++r) st[i][r] = 0.f;
     }
   }
+  if (mode == 1 && last) return;                    // (a portion of one segment: only its starting state was needed)
+  float dprod = 1.f;
 
   const float* xh = xbc + h * P;
   float* yh = y + h * P + p;
@@ -197,6 +243,7 @@ __global__ __launch_bounds__(PP == 4 ? 256 : (PP == 2 ? 512 : 1024)) void ssd_sc
     auto token = [&](int k, float (&part)[PP], float (&xs)[PP]) {
       const float* tp = lds + k * per;
       const float dt = tp[P4 + 2 * NP], dA = tp[P4 + 2 * NP + 1];
+      dprod *= dA;
       const float* Bp = (const float*)__builtin_assume_aligned(tp + P4 + g * SSD_R, 16);
       const float* Cp = (const float*)__builtin_assume_aligned(Bp + NP, 16);
       float bv[SSD_R], cv[SSD_R];
@@ -235,7 +282,7 @@ __global__ __launch_bounds__(PP == 4 ? 256 : (PP == 2 ? 512 : 1024)) void ssd_sc
               for (int i = 0; i < PP; ++i) part[k][i] += __shfl_xor(part[k][i], o, 64);
           }
         }
-        if (g == 0) {
+        if (g == 0 && mode != 1) {
 #pragma unroll
           for (int k = 0; k < SSD_SB; ++k)
 #pragma unroll
@@ -250,22 +297,18 @@ __global__ __launch_bounds__(PP == 4 ? 256 : (PP == 2 ? 512 : 1024)) void ssd_sc
         for (int i = 0; i < PP; ++i) {
           float acc = part[i];
           for (int o = NG >> 1; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
-          if (g == 0) yh[(tb + k) * inner + i] = acc + Dh * xs[i];
+          if (g == 0 && mode != 1) yh[(tb + k) * inner + i] = acc + Dh * xs[i];
         }
       }
     }
   }
+  if (mode == 1) {
 #pragma unroll
-  for (int i = 0; i < PP; ++i) {
-    if (vec) {
+    for (int i = 0; i < PP; ++i) store16(wst + (int64_t)(seg + 1) * P * N + (int64_t)i * N, st[i]);
+    if (tid == 0) wdec[seg + 1] = dprod;
+  } else if (last) {
 #pragma unroll
-      for (int r = 0; r < SSD_R; r += 4)
-        if (g * SSD_R + r < N) *(float4*)(Sh + (int64_t)i * N + r) = make_float4(st[i][r], st[i][r + 1], st[i][r + 2], st[i][r + 3]);
-    } else {
-#pragma unroll
-      for (int r = 0; r < SSD_R; ++r)
-        if (g * SSD_R + r < N) Sh[(int64_t)i * N + r] = st[i][r];
-    }
+    for (int i = 0; i < PP; ++i) store16(Sh + (int64_t)i * N, st[i]);
   }
 }
 
@@ -331,17 +374,39 @@ extern "C" int nvs_rglru_scan(const float* gates, const float* u, const void* yp
   return nvs_check_launch("nvs_rglru_scan");
 }
 
+// Segments for long portions when (portion, head) pairs alone would leave compute units idle: seg_len 0 = none.
+static void ssd_plan(int heads, int nseq, int64_t max_q, int* seg_len, int* nseg) {
+  *seg_len = 0;
+  *nseg = 1;
+  const int64_t pairs = (int64_t)heads * nseq;
+  if (pairs >= 512 || max_q < 512) return;
+  const int target = (int)((1024 + pairs - 1) / pairs);     // segments wanted per portion
+  int64_t sl = (max_q + target - 1) / target;
+  sl = (sl + 15) / 16 * 16;
+  if (sl < 128) sl = 128;
+  const int ns = (int)((max_q + sl - 1) / sl);
+  if (ns < 2) return;
+  *seg_len = (int)sl;
+  *nseg = ns;
+}
+
+extern "C" int64_t nvs_ssd_scan_workspace(int heads, int P, int N, int nseq, int64_t max_q) {
+  int seg_len, nseg;
+  ssd_plan(heads, nseq, max_q, &seg_len, &nseg);
+  return seg_len ? (int64_t)nseq * heads * (nseg + 1) * ((int64_t)P * N + 1) : 0;
+}
+
 extern "C" int nvs_ssd_scan(const float* xbc, const void* proj, int64_t proj_stride, int64_t dt_col, int dtype, const void* dt_bias,
                             const void* A_log, const void* D, int heads, int P, int N, int G, const int32_t* cu_q, const int32_t* ctx0,
-                            const int32_t* slot, int nseq, int64_t n, float* S, float* y, void* stream) {
+                            const int32_t* slot, int nseq, int64_t n, int64_t max_q, float* S, float* y, float* ws, int64_t ws_floats,
+                            void* stream) {
   NVS_REQUIRE(xbc && proj && dt_bias && A_log && D && cu_q && ctx0 && slot && S && y, "nvs_ssd_scan: null argument");
   NVS_REQUIRE(heads > 0 && G > 0 && heads % G == 0 && P > 0 && P <= 256 && N > 0 && nseq >= 0 && nseq <= 65535,
               "nvs_ssd_scan: heads %d groups %d head size %d state %d", heads, G, P, N);
   if (n == 0 || nseq == 0) return NVS_OK;
   int ng = 1;
   while (ng * SSD_R < N) ng <<= 1;                  // a power of two: the threads of one p reduce by lane shuffles
-  int ng0 = 1;
-  while (ng0 * SSD_R < N) ng0 <<= 1;
+  const int ng0 = ng;
   // Rows per thread: the 32 B / C values a thread reads from LDS per token serve PP rows, and the scan is bound by the LDS
   // pipe at PP = 1 (counters: 21 LDS instructions against 93 VALU per wavefront and token, 8 of them 16-byte reads). PP = 4
   // leaves one wavefront per SIMD and is latency-bound instead (measured slower); PP = 2 is the default where it fits.
@@ -353,18 +418,24 @@ extern "C" int nvs_ssd_scan(const float* xbc, const void* proj, int64_t proj_str
   const int threads = (P / pp) * ng, per = ((P + 3) & ~3) + 2 * ng * SSD_R + 4;
   const int tb = SSD_TB;                            // tokens per LDS round
   const size_t lds = (size_t)tb * per * sizeof(float);
-  if (pp == 2)
-    NVS_DISPATCH(dtype, ssd_scan_kernel<T, 2><<<dim3(heads, (unsigned)nseq), dim3(threads), lds, (hipStream_t)stream>>>(
-                            xbc, (const T*)proj, proj_stride, dt_col, (const T*)dt_bias, (const T*)A_log, (const T*)D, heads, P, N, G, ng,
-                            tb, cu_q, ctx0, slot, S, y));
-  else if (pp == 4)
-    NVS_DISPATCH(dtype, ssd_scan_kernel<T, 4><<<dim3(heads, (unsigned)nseq), dim3(threads), lds, (hipStream_t)stream>>>(
-                            xbc, (const T*)proj, proj_stride, dt_col, (const T*)dt_bias, (const T*)A_log, (const T*)D, heads, P, N, G, ng,
-                            tb, cu_q, ctx0, slot, S, y));
-  else
-    NVS_DISPATCH(dtype, ssd_scan_kernel<T, 1><<<dim3(heads, (unsigned)nseq), dim3(threads), lds, (hipStream_t)stream>>>(
-                            xbc, (const T*)proj, proj_stride, dt_col, (const T*)dt_bias, (const T*)A_log, (const T*)D, heads, P, N, G, ng,
-                            tb, cu_q, ctx0, slot, S, y));
+  int seg_len = 0, nseg = 1;
+  if (ws) ssd_plan(heads, nseq, max_q > 0 ? max_q : n, &seg_len, &nseg);
+  NVS_REQUIRE(!seg_len || ws_floats >= nvs_ssd_scan_workspace(heads, P, N, nseq, max_q > 0 ? max_q : n),
+              "nvs_ssd_scan: workspace of %lld floats is too small", (long long)ws_floats);
+  for (int pass = seg_len ? 1 : 0; pass <= (seg_len ? 2 : 0); ++pass) {
+    const dim3 grid(heads, (unsigned)nseq, seg_len ? nseg : 1);
+#define NVS_SSD_LAUNCH(PPV)                                                                                                         \
+  NVS_DISPATCH(dtype, ssd_scan_kernel<T, PPV><<<grid, dim3(threads), lds, (hipStream_t)stream>>>(                                    \
+                          xbc, (const T*)proj, proj_stride, dt_col, (const T*)dt_bias, (const T*)A_log, (const T*)D, heads, P, N, G, ng, \
+                          tb, cu_q, ctx0, slot, S, y, pass, seg_len, nseg, ws))
+    if (pp == 2)
+      NVS_SSD_LAUNCH(2);
+    else if (pp == 4)
+      NVS_SSD_LAUNCH(4);
+    else
+      NVS_SSD_LAUNCH(1);
+#undef NVS_SSD_LAUNCH
+  }
   return nvs_check_launch("nvs_ssd_scan");
 }
 

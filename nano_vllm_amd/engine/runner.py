@@ -964,7 +964,7 @@ class ModelRunner:
             a["rows"][nrows] = n
             nrows += 1
             n += 1
-        return dict(n=n, ns=max(len(seqs), pad_to), nrows=nrows)
+        return dict(n=n, ns=max(len(seqs), pad_to), nrows=nrows, max_q=max([s.num_scheduled_tokens for s in seqs] + [1]))
 
     def _ensure_sampler(self):
         if self.sampler is None:
@@ -1006,7 +1006,7 @@ class ModelRunner:
         st.upload()
         t = st.t
         n, ns, nrows = info["n"], info["ns"], info["nrows"]
-        por = Portions(t["cu_q"], t["ctx0"], t["sslot"], t["tseq"], ns, n)
+        por = Portions(t["cu_q"], t["ctx0"], t["sslot"], t["tseq"], ns, n, info.get("max_q", 0))
         set_context(True, slot_mapping=t["slots"][:n], block_tables=t["bt"][:ns], portions=por)
         x = self.model(t["ids"][:n], t["pos"][:n])
         logits = self.model.compute_logits(x, t["rows"], nrows)

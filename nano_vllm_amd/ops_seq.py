@@ -15,7 +15,7 @@ import torch
 
 from . import build as _build
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 _P, _I, _L, _F = c_void_p, c_int, c_int64, c_float
 
 SIGNATURES = {
@@ -27,7 +27,8 @@ SIGNATURES = {
     "nvs_xielu": (c_int, [_P, _P, _F, _I, _L, _P, _P]),
     "nvs_causal_conv": (c_int, [_P, _L, _I, _P, _P, _I, _I, _I, _P, _P, _P, _P, _I, _L, _P, _P, _P]),
     "nvs_rglru_scan": (c_int, [_P, _P, _P, _L, _I, _P, _F, _I, _I, _P, _P, _P, _I, _L, _P, _P, _P]),
-    "nvs_ssd_scan": (c_int, [_P, _P, _L, _L, _I, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _I, _L, _P, _P, _P]),
+    "nvs_ssd_scan_workspace": (c_int64, [_I, _I, _I, _I, _L]),
+    "nvs_ssd_scan": (c_int, [_P, _P, _L, _L, _I, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _I, _L, _L, _P, _P, _P, _L, _P]),
     "nvs_gated_group_norm": (c_int, [_P, _P, _L, _I, _P, _I, _I, _F, _L, _P, _P]),
     "nvs_knorm_kvstore": (c_int, [_P, _P, _L, _I, _P, _F, _I, _I, _I, _I, _P, _L, _P, _P, _P]),
     "nvs_window_attn_force_scalar": (None, [_I]),
@@ -97,10 +98,11 @@ def _same(code_of: torch.Tensor, *others: torch.Tensor | None) -> int:
 class Portions:
     """Device-side description of a step's packed portions (see include/nvl_seq.h): cu_q [nseq + 1], ctx0 [nseq],
     slot [nseq], tseq [n], all int32."""
-    __slots__ = ("cu_q", "ctx0", "slot", "tseq", "nseq", "n")
+    __slots__ = ("cu_q", "ctx0", "slot", "tseq", "nseq", "n", "max_q")
 
-    def __init__(self, cu_q, ctx0, slot, tseq, nseq: int, n: int):
+    def __init__(self, cu_q, ctx0, slot, tseq, nseq: int, n: int, max_q: int = 0):
         self.cu_q, self.ctx0, self.slot, self.tseq, self.nseq, self.n = cu_q, ctx0, slot, tseq, nseq, n
+        self.max_q = max_q or n                        # the longest portion (a host-side bound; n when unknown)
         for t in (cu_q, ctx0, slot, tseq):
             assert t.dtype == torch.int32 and t.is_cuda and t.is_contiguous()
         assert cu_q.numel() >= nseq + 1 and ctx0.numel() >= nseq and slot.numel() >= nseq and tseq.numel() >= n
@@ -179,9 +181,11 @@ def ssd_scan(xbc: torch.Tensor, proj: torch.Tensor, dt_col: int, dt_bias, A_log,
     assert S.dtype == torch.float32 and S.is_contiguous() and tuple(S.shape[1:]) == (heads, P, N)
     assert y.dtype == torch.float32 and y.is_contiguous() and y.shape == (n, inner)
     assert dt_bias.numel() == heads and A_log.numel() == heads and D.numel() == heads
+    need = 0 if torch.cuda.is_current_stream_capturing() else lib.nvs_ssd_scan_workspace(heads, P, N, por.nseq, por.max_q)
+    ws = torch.empty(need, dtype=torch.float32, device=xbc.device) if need else None
     _check(lib.nvs_ssd_scan(_ptr(xbc), _ptr(proj), proj.stride(0), dt_col, _same(proj, dt_bias, A_log, D), _ptr(dt_bias),
                             _ptr(A_log), _ptr(D), heads, P, N, G, _ptr(por.cu_q), _ptr(por.ctx0), _ptr(por.slot), por.nseq, n,
-                            _ptr(S), _ptr(y), _stream()))
+                            por.max_q, _ptr(S), _ptr(y), _ptr(ws), need, _stream()))
 
 
 def gated_group_norm(y: torch.Tensor, z: torch.Tensor, w: torch.Tensor, groups: int, eps: float, out: torch.Tensor):

@@ -519,3 +519,45 @@ def test_the_schedule_replayer_as_a_program(checkpoints, tmp_path):
     p.stdin.close()
     assert p.wait(timeout=60) == 0
     assert at == {k: len(v) for k, v in toks.items()}
+
+
+def test_state_space_recurrence_cut_into_segments_equals_the_token_loop():
+    """A long portion with few heads is scanned in segments (local states, then combined): it must equal the token loop,
+    start from the state an earlier portion left, leave the right state behind, and not disturb a short portion beside it."""
+    from nano_vllm_amd import ops_seq
+    heads, P, N, G = 2, 16, 24, 1
+    inner = heads * P
+    g = torch.Generator().manual_seed(77)
+    lens = [40, 700, 3]                                     # first call: 40 tokens of sequence A; second: 700 more of A beside 3 of B
+    TA, TB_ = 740, 3
+    def inputs(T):
+        return (torch.randn(T, inner + 2 * G * N, generator=g), torch.randn(T, heads, generator=g))
+    (xa, pa), (xb, pb) = inputs(TA), inputs(TB_)
+    dt_bias, A_log, D = torch.randn(heads, generator=g) - 3, torch.randn(heads, generator=g) - 2, torch.randn(heads, generator=g)
+
+    def loop(xbc, proj):
+        T = xbc.shape[0]
+        x, B, C = xbc[:, :inner].double().view(T, heads, P), xbc[:, inner:inner + N].double(), xbc[:, inner + N:].double()
+        dt = plain.softplus(proj.double() + dt_bias.double())
+        S = torch.zeros(heads, N, P, dtype=F64)
+        y = torch.zeros(T, heads, P, dtype=F64)
+        for t in range(T):
+            for h in range(heads):
+                S[h] = torch.exp(-torch.exp(A_log[h].double()) * dt[t, h]) * S[h] + dt[t, h] * torch.outer(B[t], x[t, h])
+                y[t, h] = S[h].T @ C[t] + D[h].double() * x[t, h]
+        return y.reshape(T, inner), S
+    (ya, Sa), (yb, Sb) = loop(xa, pa), loop(xb, pb)
+    state = torch.full((3, heads, P, N), 9.0, device="cuda")
+    y0 = torch.empty(40, inner, device="cuda")
+    ops_seq.ssd_scan(dev(xa[:40]), dev(pa[:40]), 0, dev(dt_bias), dev(A_log), dev(D), heads, P, N, G, portions([40], [0], [2]), state, y0)
+    por = portions([700, 3], [40, 0], [2, 0])
+    por.max_q = 700
+    assert ops_seq.load_library().nvs_ssd_scan_workspace(heads, P, N, 2, 700) > 0, "this shape was meant to be segmented"
+    y1 = torch.empty(703, inner, device="cuda")
+    ops_seq.ssd_scan(dev(torch.cat([xa[40:], xb])), dev(torch.cat([pa[40:], pb])), 0, dev(dt_bias), dev(A_log), dev(D), heads, P, N, G,
+                     por, state, y1)
+    close(torch.cat([y0, y1[:700]]), ya, 3e-5, "long sequence")
+    close(y1[700:], yb, 3e-5, "short neighbour")
+    close(state[2].transpose(1, 2), Sa, 3e-5, "state of the long sequence")
+    close(state[0].transpose(1, 2), Sb, 3e-5, "state of the short one")
+    assert (state[1] == 9).all()
