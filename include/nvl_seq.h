@@ -60,10 +60,13 @@ int nvs_causal_conv(const void* in, int64_t in_stride, int dtype, const void* w,
  * (first bw) and of the input gate (last bw), biases included; u [n, C] 32-bit; ypre [n, C] (row stride y_stride) the
  * pre-activation of the output branch (GELU-tanh is applied here); lam [C]. For every channel, token by token:
  *   a = exp(-c * sigmoid(gr) * softplus(lam)),  S = a S + sqrt(1 - a^2) * sigmoid(gi) * u,  out = S * gelu_tanh(ypre).
- * S [nslots, C] 32-bit, advanced. out [n, C] `dtype`. */
+ * S [nslots, C] 32-bit, advanced. out [n, C] `dtype`. Long portions of a step with few (portion, channel) threads are scanned
+ * in segments, twice, in `ws` (nvs_rglru_scan_workspace floats; NULL: never), as nvs_ssd_scan below explains; max_q = the
+ * longest portion of the step. */
+int64_t nvs_rglru_scan_workspace(int channels, int nseq, int64_t max_q);
 int nvs_rglru_scan(const float* gates, const float* u, const void* ypre, int64_t y_stride, int dtype, const void* lam, float c,
                    int channels, int blocks, const int32_t* cu_q, const int32_t* ctx0, const int32_t* slot, int nseq, int64_t n,
-                   float* S, void* out, void* stream);
+                   int64_t max_q, float* S, void* out, float* ws, int64_t ws_floats, void* stream);
 
 /* State-space-duality recurrence, recurrent form. xbc [n, inner + 2*G*N] 32-bit (x | B | C after convolution + SiLU),
  * dt: column dt_col .. dt_col + heads of proj [n, proj_stride] (`dtype`); dt_bias, A_log, D [heads] (`dtype`). Per head h

@@ -72,36 +72,83 @@ __global__ void conv_state_kernel(const T* __restrict__ in, int64_t in_stride, i
 }
 
 // ---- real-gated linear recurrence ---------------------------------------------------------------------------------
-// one thread per (portion, channel), sequential over the portion's tokens; loads do not depend on the recurrence, so the
-// compiler keeps several tokens' operands in flight
+// One thread per (portion, channel), sequential over the portion's tokens; loads do not depend on the recurrence, so the
+// compiler keeps several tokens' operands in flight. Long portions of a step with few (portion, channel) threads are cut
+// into segments of seg_len tokens (blockIdx.z) and scanned twice, as the SSD scan below does:
+//   mode 1: every segment but a portion's last from zero -> its final value L_k and decay product d_k to `ws`
+//           ([nseq][nseg + 1][2][channels]; entry 0 holds the value the portion starts from);
+//   mode 2: segment k starts from S_k = d_(k-1) S_(k-1) + L_(k-1) and writes the outputs; the last one writes the slot.
 template <typename T>
 __global__ void rglru_scan_kernel(const float* __restrict__ gates, const float* __restrict__ u, const T* __restrict__ ypre,
                                   int64_t y_stride, const T* __restrict__ lam, float cmul, int channels, int blocks,
                                   const int32_t* __restrict__ cu_q, const int32_t* __restrict__ ctx0,
-                                  const int32_t* __restrict__ slot, int64_t n, float* __restrict__ S, T* __restrict__ out) {
-  const int s = blockIdx.y;
+                                  const int32_t* __restrict__ slot, int64_t n, float* __restrict__ S, T* __restrict__ out, int mode,
+                                  int seg_len, int nseg, float* __restrict__ ws) {
+  const int s = blockIdx.y, seg = blockIdx.z;
   const int c = blockIdx.x * blockDim.x + threadIdx.x;
   if (c >= channels) return;
-  const int64_t q0 = cu_q[s], q1 = cu_q[s + 1];
+  const int64_t p0 = cu_q[s], p1 = cu_q[s + 1];
+  const int64_t q0 = mode == 0 ? p0 : p0 + (int64_t)seg * seg_len;
+  const int64_t q1 = mode == 0 ? p1 : (q0 + seg_len < p1 ? q0 + seg_len : p1);
   if (q1 <= q0) return;
+  const bool last = q1 == p1;
   const int bw = channels / blocks, blk = c / bw, cc = c - blk * bw;
   const float sp = softplusf_(ldf(lam + c));
   float* sp_state = S + (int64_t)slot[s] * channels + c;
-  float st = ctx0[s] == 0 ? 0.f : *sp_state;
+  float* wv = ws + ((int64_t)s * (nseg + 1)) * 2 * channels + c;          // entry e: value at + 2 e C, decay at + (2 e + 1) C
+  float st = 0.f;
+  if (mode == 2) {
+    st = wv[0];
+    for (int k = 0; k < seg; ++k) st = wv[(int64_t)(2 * k + 3) * channels] * st + wv[(int64_t)(2 * k + 2) * channels];
+  } else if (ctx0[s] != 0 && (mode == 0 || seg == 0)) {
+    st = *sp_state;
+  }
+  if (mode == 1) {
+    if (seg == 0) wv[0] = st;
+    if (last) return;
+    st = 0.f;
+  }
+  float dsum = 0.f;                                 // sum of log a over the segment
   const float* gp = gates + ((int64_t)blk * n) * (2 * bw) + cc;
 #pragma unroll 4
   for (int64_t t = q0; t < q1; ++t) {
     const float gr = gp[t * (2 * bw)], gi = gp[t * (2 * bw) + bw];
     const float uv = u[t * channels + c];
-    const float yv = gelu_tanhf_(ldf(ypre + t * y_stride + c));
     const float r = 1.f / (1.f + expf(-gr)), ig = 1.f / (1.f + expf(-gi));
     const float log_a = -cmul * r * sp;
     const float a = expf(log_a);
     const float mult = sqrtf(fmaxf(-expm1f(2.f * log_a), 0.f));     // sqrt(1 - a^2), without cancellation near a = 1
     st = a * st + mult * (ig * uv);
-    stf(out + t * channels + c, st * yv);
+    dsum += log_a;
+    if (mode != 1) stf(out + t * channels + c, st * gelu_tanhf_(ldf(ypre + t * y_stride + c)));
   }
-  *sp_state = st;
+  if (mode == 1) {
+    wv[(int64_t)(2 * seg + 2) * channels] = st;
+    wv[(int64_t)(2 * seg + 3) * channels] = expf(dsum);
+  } else if (last) {
+    *sp_state = st;
+  }
+}
+
+// Segments for the elementwise recurrence: seg_len 0 = none.
+static void rglru_plan(int channels, int nseq, int64_t max_q, int* seg_len, int* nseg) {
+  *seg_len = 0;
+  *nseg = 1;
+  const int64_t threads = (int64_t)channels * nseq;
+  if (threads >= 131072 || max_q < 512) return;    // two wavefronts per SIMD already, or nothing to cut
+  const int target = (int)((131072 + threads - 1) / threads);
+  int64_t sl = (max_q + target - 1) / target;
+  if (sl < 64) sl = 64;
+  const int ns = (int)((max_q + sl - 1) / sl);
+  if (ns < 2) return;
+  *seg_len = (int)sl;
+  *nseg = ns;
+}
+
+extern "C" int64_t nvs_rglru_scan_workspace(int channels, int nseq, int64_t max_q) {
+  int seg_len, nseg;
+  rglru_plan(channels, nseq, max_q, &seg_len, &nseg);
+  return seg_len ? (int64_t)nseq * (nseg + 1) * 2 * channels : 0;
 }
 
 // ---- state-space-duality recurrence -------------------------------------------------------------------------------
@@ -363,14 +410,20 @@ extern "C" int nvs_causal_conv(const void* in, int64_t in_stride, int dtype, con
 
 extern "C" int nvs_rglru_scan(const float* gates, const float* u, const void* ypre, int64_t y_stride, int dtype, const void* lam,
                               float c, int channels, int blocks, const int32_t* cu_q, const int32_t* ctx0, const int32_t* slot, int nseq,
-                              int64_t n, float* S, void* out, void* stream) {
+                              int64_t n, int64_t max_q, float* S, void* out, float* ws, int64_t ws_floats, void* stream) {
   NVS_REQUIRE(gates && u && ypre && lam && cu_q && ctx0 && slot && S && out, "nvs_rglru_scan: null argument");
   NVS_REQUIRE(channels > 0 && blocks > 0 && channels % blocks == 0 && y_stride >= channels && nseq >= 0 && nseq <= 65535 && n >= 0,
               "nvs_rglru_scan: channels %d blocks %d", channels, blocks);
   if (n == 0 || nseq == 0) return NVS_OK;
+  int seg_len = 0, nseg = 1;
+  if (ws) rglru_plan(channels, nseq, max_q > 0 ? max_q : n, &seg_len, &nseg);
+  NVS_REQUIRE(!seg_len || ws_floats >= nvs_rglru_scan_workspace(channels, nseq, max_q > 0 ? max_q : n),
+              "nvs_rglru_scan: workspace of %lld floats is too small", (long long)ws_floats);
   const dim3 block(64);
-  NVS_DISPATCH(dtype, rglru_scan_kernel<T><<<dim3((channels + 63) / 64, (unsigned)nseq), block, 0, (hipStream_t)stream>>>(
-                          gates, u, (const T*)ypre, y_stride, (const T*)lam, c, channels, blocks, cu_q, ctx0, slot, n, S, (T*)out));
+  for (int pass = seg_len ? 1 : 0; pass <= (seg_len ? 2 : 0); ++pass)
+    NVS_DISPATCH(dtype, rglru_scan_kernel<T><<<dim3((channels + 63) / 64, (unsigned)nseq, seg_len ? nseg : 1), block, 0, (hipStream_t)stream>>>(
+                            gates, u, (const T*)ypre, y_stride, (const T*)lam, c, channels, blocks, cu_q, ctx0, slot, n, S, (T*)out, pass,
+                            seg_len, nseg, ws));
   return nvs_check_launch("nvs_rglru_scan");
 }
 

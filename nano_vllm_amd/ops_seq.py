@@ -26,7 +26,8 @@ SIGNATURES = {
     "nvs_scalar_norm_rows": (c_int, [_P, _P, _L, _I, _P, _I, _F, _P, _P]),
     "nvs_xielu": (c_int, [_P, _P, _F, _I, _L, _P, _P]),
     "nvs_causal_conv": (c_int, [_P, _L, _I, _P, _P, _I, _I, _I, _P, _P, _P, _P, _I, _L, _P, _P, _P]),
-    "nvs_rglru_scan": (c_int, [_P, _P, _P, _L, _I, _P, _F, _I, _I, _P, _P, _P, _I, _L, _P, _P, _P]),
+    "nvs_rglru_scan_workspace": (c_int64, [_I, _I, _L]),
+    "nvs_rglru_scan": (c_int, [_P, _P, _P, _L, _I, _P, _F, _I, _I, _P, _P, _P, _I, _L, _L, _P, _P, _P, _L, _P]),
     "nvs_ssd_scan_workspace": (c_int64, [_I, _I, _I, _I, _L]),
     "nvs_ssd_scan": (c_int, [_P, _P, _L, _L, _I, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _I, _L, _L, _P, _P, _P, _L, _P]),
     "nvs_gated_group_norm": (c_int, [_P, _P, _L, _I, _P, _I, _I, _F, _L, _P, _P]),
@@ -167,8 +168,11 @@ def rglru_scan(gates: torch.Tensor, u: torch.Tensor, ypre: torch.Tensor, lam: to
     assert u.dtype == torch.float32 and u.is_contiguous() and ypre.shape == (n, channels) and ypre.stride(1) == 1
     assert S.dtype == torch.float32 and S.is_contiguous() and S.shape[1] == channels and lam.numel() == channels
     assert out.shape == (n, channels) and out.is_contiguous()
+    need = 0 if torch.cuda.is_current_stream_capturing() else lib.nvs_rglru_scan_workspace(channels, por.nseq, por.max_q)
+    ws = torch.empty(need, dtype=torch.float32, device=u.device) if need else None
     _check(lib.nvs_rglru_scan(_ptr(gates), _ptr(u), _ptr(ypre), ypre.stride(0), _same(ypre, lam, out), _ptr(lam), c, channels,
-                              blocks, _ptr(por.cu_q), _ptr(por.ctx0), _ptr(por.slot), por.nseq, n, _ptr(S), _ptr(out), _stream()))
+                              blocks, _ptr(por.cu_q), _ptr(por.ctx0), _ptr(por.slot), por.nseq, n, por.max_q, _ptr(S), _ptr(out), _ptr(ws), need,
+                              _stream()))
 
 
 def ssd_scan(xbc: torch.Tensor, proj: torch.Tensor, dt_col: int, dt_bias, A_log, D, heads: int, P: int, N: int, G: int,

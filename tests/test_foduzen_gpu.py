@@ -561,3 +561,35 @@ def test_state_space_recurrence_cut_into_segments_equals_the_token_loop():
     close(state[2].transpose(1, 2), Sa, 3e-5, "state of the long sequence")
     close(state[0].transpose(1, 2), Sb, 3e-5, "state of the short one")
     assert (state[1] == 9).all()
+
+
+def test_gated_recurrence_cut_into_segments_equals_the_token_loop():
+    """A long portion of a narrow layer is scanned in segments; beside it a short portion of another sequence that continues
+    from a stored state."""
+    from nano_vllm_amd import ops_seq
+    g = torch.Generator().manual_seed(6)
+    C, blocks, T, T2 = 40, 2, 1500, 3
+    bw = C // blocks
+    p = {"ra": torch.randn(blocks, bw, bw, generator=g) * 0.2, "ra.b": torch.randn(blocks, bw, generator=g),
+         "ri": torch.randn(blocks, bw, bw, generator=g) * 0.2, "ri.b": torch.randn(blocks, bw, generator=g),
+         "lam": -8.0 + 6 * torch.rand(C, generator=g)}
+    pd = {k: v.double() for k, v in p.items()}
+    u, ypre = torch.randn(T + T2, C, generator=g), torch.randn(T + T2, C, generator=g)
+    s2 = torch.randn(C, generator=g)                                      # what the second sequence's slot holds
+    want1, S1 = plain.rglru(u[:T].double(), plain.gelu_tanh(ypre[:T].double()), pd, blocks, torch.zeros(C, dtype=F64))
+    want2, S2 = plain.rglru(u[T:].double(), plain.gelu_tanh(ypre[T:].double()), pd, blocks, s2.double())
+    ub = u.double().view(T + T2, blocks, bw)
+    gr = torch.einsum("boi,tbi->bto", pd["ra"], ub) + pd["ra.b"][:, None]
+    gi = torch.einsum("boi,tbi->bto", pd["ri"], ub) + pd["ri.b"][:, None]
+    state = torch.full((3, C), -9.0, device="cuda")
+    state[0] = dev(s2)
+    por = portions([T, T2], [0, 17], [2, 0])
+    por.max_q = T
+    assert ops_seq.load_library().nvs_rglru_scan_workspace(C, 2, T) > 0, "this shape was meant to be segmented"
+    out = torch.empty(T + T2, C, device="cuda")
+    ops_seq.rglru_scan(dev(torch.cat([gr, gi], -1).float()), dev(u), dev(ypre), dev(p["lam"]), 8.0, blocks, por, state, out)
+    close(out[:T], want1, 3e-5, "long sequence")
+    close(out[T:], want2, 3e-5, "short neighbour")
+    close(state[2], S1, 3e-5, "state of the long sequence")
+    close(state[0], S2, 3e-5, "state of the short one")
+    assert (state[1] == -9).all()
