@@ -78,12 +78,13 @@ __global__ void conv_state_kernel(const T* __restrict__ in, int64_t in_stride, i
 //   mode 1: every segment but a portion's last from zero -> its final value L_k and decay product d_k to `ws`
 //           ([nseq][nseg + 1][2][channels]; entry 0 holds the value the portion starts from);
 //   mode 2: segment k starts from S_k = d_(k-1) S_(k-1) + L_(k-1) and writes the outputs; the last one writes the slot.
-template <typename T>
+template <typename T, int MODE>
 __global__ void rglru_scan_kernel(const float* __restrict__ gates, const float* __restrict__ u, const T* __restrict__ ypre,
                                   int64_t y_stride, const T* __restrict__ lam, float cmul, int channels, int blocks,
                                   const int32_t* __restrict__ cu_q, const int32_t* __restrict__ ctx0,
-                                  const int32_t* __restrict__ slot, int64_t n, float* __restrict__ S, T* __restrict__ out, int mode,
-                                  int seg_len, int nseg, float* __restrict__ ws) {
+                                  const int32_t* __restrict__ slot, int64_t n, float* __restrict__ S, T* __restrict__ out, int seg_len,
+                                  int nseg, float* __restrict__ ws) {
+  constexpr int mode = MODE;                        // (compile-time: the plain scan keeps its straight-line loop)
   const int s = blockIdx.y, seg = blockIdx.z;
   const int c = blockIdx.x * blockDim.x + threadIdx.x;
   if (c >= channels) return;
@@ -160,12 +161,13 @@ constexpr int SSD_R = 16;      // state entries per thread
 constexpr int SSD_TB = 16;     // tokens per LDS round
 constexpr int SSD_SB = 8;      // tokens whose cross-lane sums are taken together
 
-template <typename T, int PP>     // PP head-size entries per thread: the B / C values read from LDS serve PP state rows
+template <typename T, int PP, int MODE>     // PP head-size entries per thread: the B / C values read from LDS serve PP state rows
 __global__ __launch_bounds__(PP == 4 ? 256 : (PP == 2 ? 512 : 1024)) void ssd_scan_kernel(const float* __restrict__ xbc, const T* __restrict__ proj, int64_t proj_stride, int64_t dt_col,
                                 const T* __restrict__ dt_bias, const T* __restrict__ A_log, const T* __restrict__ Dp, int heads,
                                 int P, int N, int G, int NG, int TB, const int32_t* __restrict__ cu_q,
                                 const int32_t* __restrict__ ctx0, const int32_t* __restrict__ slot, float* __restrict__ S,
-                                float* __restrict__ y, int mode, int seg_len, int nseg, float* __restrict__ ws) {
+                                float* __restrict__ y, int seg_len, int nseg, float* __restrict__ ws) {
+  constexpr int mode = MODE;                        // (compile-time: the unsegmented scan pays nothing for the other two)
   // mode 0: the whole portion in one workgroup. Long portions with few (portion, head) pairs are cut into segments of
   // seg_len tokens (blockIdx.z) and scanned twice, because one workgroup walks its tokens one after the other:
   //   mode 1: every segment but a portion's last from a ZERO state -> its final state L_k and decay product d_k to `ws`
@@ -420,10 +422,17 @@ extern "C" int nvs_rglru_scan(const float* gates, const float* u, const void* yp
   NVS_REQUIRE(!seg_len || ws_floats >= nvs_rglru_scan_workspace(channels, nseq, max_q > 0 ? max_q : n),
               "nvs_rglru_scan: workspace of %lld floats is too small", (long long)ws_floats);
   const dim3 block(64);
-  for (int pass = seg_len ? 1 : 0; pass <= (seg_len ? 2 : 0); ++pass)
-    NVS_DISPATCH(dtype, rglru_scan_kernel<T><<<dim3((channels + 63) / 64, (unsigned)nseq, seg_len ? nseg : 1), block, 0, (hipStream_t)stream>>>(
-                            gates, u, (const T*)ypre, y_stride, (const T*)lam, c, channels, blocks, cu_q, ctx0, slot, n, S, (T*)out, pass,
-                            seg_len, nseg, ws));
+#define NVS_RGLRU_LAUNCH(MODE)                                                                                                     \
+  NVS_DISPATCH(dtype, rglru_scan_kernel<T, MODE><<<dim3((channels + 63) / 64, (unsigned)nseq, seg_len ? nseg : 1), block, 0,         \
+                                                  (hipStream_t)stream>>>(gates, u, (const T*)ypre, y_stride, (const T*)lam, c, channels, \
+                                                                         blocks, cu_q, ctx0, slot, n, S, (T*)out, seg_len, nseg, ws))
+  if (seg_len) {
+    NVS_RGLRU_LAUNCH(1);
+    NVS_RGLRU_LAUNCH(2);
+  } else {
+    NVS_RGLRU_LAUNCH(0);
+  }
+#undef NVS_RGLRU_LAUNCH
   return nvs_check_launch("nvs_rglru_scan");
 }
 
@@ -477,20 +486,27 @@ extern "C" int nvs_ssd_scan(const float* xbc, const void* proj, int64_t proj_str
   if (ws) ssd_plan(heads, nseq, max_q > 0 ? max_q : n, &seg_len, &nseg);
   NVS_REQUIRE(!seg_len || ws_floats >= nvs_ssd_scan_workspace(heads, P, N, nseq, max_q > 0 ? max_q : n),
               "nvs_ssd_scan: workspace of %lld floats is too small", (long long)ws_floats);
-  for (int pass = seg_len ? 1 : 0; pass <= (seg_len ? 2 : 0); ++pass) {
-    const dim3 grid(heads, (unsigned)nseq, seg_len ? nseg : 1);
-#define NVS_SSD_LAUNCH(PPV)                                                                                                         \
-  NVS_DISPATCH(dtype, ssd_scan_kernel<T, PPV><<<grid, dim3(threads), lds, (hipStream_t)stream>>>(                                    \
+  const dim3 grid(heads, (unsigned)nseq, seg_len ? nseg : 1);
+#define NVS_SSD_LAUNCH(PPV, MODE)                                                                                                   \
+  NVS_DISPATCH(dtype, ssd_scan_kernel<T, PPV, MODE><<<grid, dim3(threads), lds, (hipStream_t)stream>>>(                              \
                           xbc, (const T*)proj, proj_stride, dt_col, (const T*)dt_bias, (const T*)A_log, (const T*)D, heads, P, N, G, ng, \
-                          tb, cu_q, ctx0, slot, S, y, pass, seg_len, nseg, ws))
-    if (pp == 2)
-      NVS_SSD_LAUNCH(2);
-    else if (pp == 4)
-      NVS_SSD_LAUNCH(4);
-    else
-      NVS_SSD_LAUNCH(1);
-#undef NVS_SSD_LAUNCH
+                          tb, cu_q, ctx0, slot, S, y, seg_len, nseg, ws))
+#define NVS_SSD_PASSES(PPV)   \
+  if (seg_len) {              \
+    NVS_SSD_LAUNCH(PPV, 1);   \
+    NVS_SSD_LAUNCH(PPV, 2);   \
+  } else {                    \
+    NVS_SSD_LAUNCH(PPV, 0);   \
   }
+  if (pp == 2) {
+    NVS_SSD_PASSES(2)
+  } else if (pp == 4) {
+    NVS_SSD_PASSES(4)
+  } else {
+    NVS_SSD_PASSES(1)
+  }
+#undef NVS_SSD_PASSES
+#undef NVS_SSD_LAUNCH
   return nvs_check_launch("nvs_ssd_scan");
 }
 
