@@ -30,7 +30,7 @@ int nvs_abi_version(void);
 const char* nvs_last_error(void);
 
 /* x[t, :] = table[ids[t], :] * scale + sinusoid(pos[t]); entry 2i = sin(pos * base^(-2i/width)), 2i+1 = cos of the same
- * angle (angles in 32-bit from an exact integer position). xh (nullable): copy of x in `dtype`. */
+ * angle (angles in 32-bit from an exact integer position); base == 0: no sinusoid. xh (nullable): copy of x in `dtype`. */
 int nvs_embed_sinusoid(const void* table, int dtype, const int64_t* ids, const int64_t* pos, int64_t n, int width,
                        float scale, float base, float* x, void* xh, void* stream);
 
@@ -39,6 +39,13 @@ int nvs_embed_sinusoid(const void* table, int dtype, const int64_t* ids, const i
  * m' = (rms(m) * w1 + rms(m2) * w2) / 2, x += g * rms(m'). rms(v) = v / sqrt(mean(v^2) + eps). xh (nullable): x in `dtype`. */
 int nvs_norm_residual(const void* m, const void* m2, const void* w1, const void* w2, const void* g, int dtype, int64_t n,
                       int width, float eps, float* x, void* xh, void* stream);
+
+/* Input-side norm on the residual stream, with the adds that precede it: x[t, :] += a[t, :] + b[t, :] (a in `dtype`, b 32-bit,
+ * either may be NULL), then out[t, :] = group_rms(x[t, :]) * w: every one of `groups` equal consecutive parts of the row is
+ * divided by its own sqrt(mean(part^2) + eps). out == NULL: the adds only. With rows != NULL nothing is added and
+ * out[r, :] is the norm of x[rows[r], :]. out and w in `dtype`. */
+int nvs_add_group_norm(float* x, const void* a, const float* b, const int32_t* rows, int64_t nrows, const void* w, int dtype,
+                       int width, int groups, float eps, void* out, void* stream);
 
 /* out[r, :] = g * rms(x[rows[r], :]) in `dtype` (rows == NULL: row r). */
 int nvs_scalar_norm_rows(const float* x, const int32_t* rows, int64_t nrows, int width, const void* g, int dtype, float eps,
@@ -81,30 +88,75 @@ int nvs_ssd_scan(const float* xbc, const void* proj, int64_t proj_stride, int64_
                  const int32_t* slot, int nseq, int64_t n, int64_t max_q, float* S, float* y, float* ws, int64_t ws_floats,
                  void* stream);
 
-/* out = group_rms(y * silu(z)) * w: the gate first, then each of `groups` equal parts of a row by its own root mean square.
- * y [n, inner] 32-bit; z [n, inner] with row stride z_stride (`dtype`); w [inner]; out [n, inner] `dtype`. */
-int nvs_gated_group_norm(const float* y, const void* z, int64_t z_stride, int dtype, const void* w, int inner, int groups,
-                         float eps, int64_t n, void* out, void* stream);
+/* The decaying outer-product recurrence of linear ("lightning") attention, in 32-bit: per head h, token by token,
+ *   S = decay[h] S + k v^T,  o = S^T q,  with q, k (dk per head) and v (dv per head) = SiLU of columns q_col / k_col / v_col
+ * (+ head * size) of proj [n, proj_stride] (`dtype`); SiLU is applied here. decay [heads] 32-bit. State memory is
+ * [nslots, heads, dv, dk] (dk fastest), advanced. y [n, heads * dv] 32-bit. The walk, the segments for long portions and the
+ * workspace (nvs_ssd_scan_workspace(heads, dv, dk, nseq, max_q)) are those of nvs_ssd_scan. */
+int nvs_decay_scan(const void* proj, int64_t proj_stride, int64_t v_col, int64_t k_col, int64_t q_col, int dtype, const float* decay,
+                   int heads, int dk, int dv, const int32_t* cu_q, const int32_t* ctx0, const int32_t* slot, int nseq, int64_t n,
+                   int64_t max_q, float* S, float* y, float* ws, int64_t ws_floats, void* stream);
 
-/* Key norm + paged K/V store. k [n, G, d] / v [n, G, dv] are column ranges of one projection output (row stride `stride`,
+/* order 0: out = group_rms(y * silu(z)) * w: the gate first, then each of `groups` equal parts of a row by its own root mean
+ * square. order 1: out = group_rms(y) * w * sigmoid(z): the norm first. y [n, inner] 32-bit; z [n, inner] with row stride z_stride
+ * (`dtype`); w [inner]; out [n, inner] `dtype`. */
+int nvs_gated_group_norm(const float* y, const void* z, int64_t z_stride, int dtype, const void* w, int inner, int groups,
+                         float eps, int order, int64_t n, void* out, void* stream);
+
+/* Key norm / rotation + paged K/V store. Rotation (rot_dims > 0, after the norm): entries (2i, 2i+1), i < rot_dims / 2, of every key head turn by
+ * the angle pos[t] * rot_freq[i] (32-bit): (u, v) -> (u cos - v sin, v cos + u sin); the other entries pass. k [n, G, d] / v [n, G, dv] are column ranges of one projection output (row stride `stride`,
  * `dtype`). k is RMS-normed over d with weight knorm [d] (NULL: stored as is). Token t goes to cache slot slots[t] (< 0:
  * skipped); slot = page * block_size + offset. Caches, `dtype`: k_cache [slot][G][d]; v_cache [page][G][dv][block_size] — values
  * are kept TRANSPOSED inside a page, so that a column's consecutive tokens are contiguous (the matrix-core attention reads 8 at a
  * time). */
 int nvs_knorm_kvstore(const void* k, const void* v, int64_t stride, int dtype, const void* knorm, float eps, int G, int d, int dv,
-                      int block_size, const int32_t* slots, int64_t n, void* k_cache, void* v_cache, void* stream);
+                      int block_size, const int32_t* slots, const int64_t* pos, const float* rot_freq, int rot_dims, int64_t n,
+                      void* k_cache, void* v_cache, void* stream);
 
-/* Sliding-window softmax attention over the paged cache, one query per token row, any d, dv <= 256.
- * q [n, H, d] (row stride q_stride), RMS-normed per head with qnorm [d] here (NULL: none). Token t of portion s sits at position
- * p = ctx0[s] + (t - cu_q[s]) and sees keys j with 0 <= p - j < window (window <= 0: every j <= p), read through
- * block_tables [nseq, bt_stride]. score = q.k * scale, ordinary softmax in 32-bit. gate (nullable) [n, H*dv] with row stride
+/* Locally masked softmax attention over the paged cache, one query per token row, any d, dv <= 256.
+ * q [n, H, d] (row stride q_stride), RMS-normed per head with qnorm [d] here (NULL: none), then rotated like the keys
+ * (rot_dims, rot_freq; 0: not). Token t of portion s sits at position p = ctx0[s] + (t - cu_q[s]) and sees keys j with
+ * 0 <= p - j < window (window > 0), or the keys j <= p of its own block, floor(j / chunk) == floor(p / chunk) (chunk > 0; blocks
+ * are counted from position 0 of the sequence), or every j <= p (both 0), read through block_tables [nseq, bt_stride]. score = q.k * scale, ordinary softmax in 32-bit. gate (nullable) [n, H*dv] with row stride
  * gate_stride: out *= sigmoid(gate). out [n, H*dv] `dtype`.
  * bf16 with d % 8 == 0 and block_size % 8 == 0 runs on the matrix cores (16 queries per wavefront; the weights enter the
  * second product as bf16); everything else, and every float32 call, takes the scalar kernel (one wavefront per query). */
 int nvs_window_attn(const void* q, int64_t q_stride, const void* qnorm, float eps, const void* gate, int64_t gate_stride, int dtype,
                     const void* k_cache, const void* v_cache, const int32_t* block_tables, int64_t bt_stride, int block_size,
                     const int32_t* cu_q, const int32_t* ctx0, const int32_t* tseq, int nseq, int64_t n, int H, int G, int d, int dv,
-                    float scale, int window, void* out, void* stream);
+                    float scale, int window, int chunk, const float* rot_freq, int rot_dims, void* out, void* stream);
+
+/* Gated feed-forward activation on a fused [gate | up] projection: gu [n, 2 ff] with row stride `stride` -> out [n, ff] (`dtype`).
+ * kind 0: silu(g) u. kind 1: g' = min(g, limit), u' = clamp(u, -limit, limit), out = g' sigmoid(alpha g') (u' + 1). */
+int nvs_glu_act(const void* gu, int64_t stride, int dtype, int ff, int kind, float limit, float alpha, int64_t n, void* out, void* stream);
+
+/* Routing of a mixture of experts, 32-bit. z [n, total] (row stride z_stride): router logits of all `total` entries.
+ * s = softmax(z); choice score c = s + correction (NULL: none). Entries form `count` equal groups of neighbours; a group's score
+ * is its largest c, and only entries of the `keep` best groups can be chosen. The `top` entries with the largest c are chosen:
+ * ids [n, top]; wts [n, top] = s[chosen] / (sum of them + 1e-20) * scale. Ties go to the lower index. */
+int nvs_moe_route(const float* z, int64_t z_stride, const float* correction, int64_t n, int total, int top, int count, int keep, float scale,
+                  int32_t* ids, float* wts, void* stream);
+
+/* Sort the pairs (token, choice) by expert. Pairs whose id >= experts have no rows (pass-through entries). Every expert's rows are
+ * padded to whole tiles of tm (16 or 64) rows; cap = nvs_moe_rows(n * top, experts, tm) rows are laid out.
+ * tile_expert [cap / tm]: the tile's expert or -1; row_token [cap]: the row's token or -1; pair_row [n * top]: the pair's row or -1. */
+int64_t nvs_moe_rows(int64_t pairs, int experts, int tm);
+int nvs_moe_plan(const int32_t* ids, int64_t n, int top, int experts, int tm, int32_t* tile_expert, int32_t* row_token, int32_t* pair_row,
+                 void* stream);
+
+/* Grouped product over the planned rows: out[r, :] = W[expert of r] x(r). glu != 0: W [experts, 2 nout, K] (gate rows, then up rows),
+ * x(r) = X[row_token[r], :], out = silu(gate) * up; glu == 0: W [experts, nout, K], x(r) = X[r, :]. X, W, out in `dtype`; bf16 with
+ * K % 8 == 0 and ldx % 8 == 0 runs on the matrix cores. Padding rows are not written. */
+int nvs_moe_gemm(const void* X, int64_t ldx, const void* W, int dtype, int glu, int nout, int K, const int32_t* tile_expert,
+                 const int32_t* row_token, int64_t cap, int tm, void* out, int64_t ldo, void* stream);
+/* tests: 1 routes bf16 calls through the plain kernel as well */
+void nvs_moe_force_plain(int on);
+
+/* out[t, :] = sum_k wts[t, k] * (pair_row[t, k] >= 0 ? rows[pair_row[t, k], :] : h[t, :]) + sigmoid(shared_gate[t]) * shared[t, :]
+ * (shared NULL: no shared expert; shared_gate 32-bit pre-activations with row stride gate_stride). */
+int nvs_moe_combine(const void* rows, int64_t ldr, const int32_t* pair_row, const float* wts, int top, const void* h, int64_t ldh,
+                    const void* shared, const float* shared_gate, int64_t gate_stride, int dtype, int64_t n, int width, void* out,
+                    void* stream);
 
 /* Tests and A/B runs: 1 routes bf16 calls through the scalar kernel too; 2 keeps the matrix-core kernel but without sharing
  * K / V tiles through LDS; 0 restores the defaults. */

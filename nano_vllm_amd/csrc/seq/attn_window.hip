@@ -1,16 +1,26 @@
-// Paged attention with a sliding window for any head size: key norm + K/V store, and the attention itself (one wavefront
+// Paged attention with a local mask for any head size: key norm / rotation + K/V store, and the attention itself (one wavefront
 // per (token row, query head): portions of prompts and single decoded tokens are the same launch). Scores, softmax and the
-// output accumulation are 32-bit; the query norm and the sigmoid output gate are fused in.
+// output accumulation are 32-bit; the query norm, the rotation of the query and the sigmoid output gate are fused in.
+// The mask is one of: a sliding window (the last `window` positions), blocks (`chunk` > 0: a query sees the keys of its own
+// block of `chunk` positions, blocks counted from position 0 of the sequence), or plain causal.
 #include "seq_common.h"
 
 namespace {
 
 constexpr int MAX_HEAD = 256;
 
+// first key position the query at position p sees (both masks are monotone in p, which the tile bounds below rely on)
+__device__ __forceinline__ int vis_lo(int p, int window, int chunk) {
+  if (window > 0) return p - window + 1 > 0 ? p - window + 1 : 0;
+  if (chunk > 0) return p - p % chunk;
+  return 0;
+}
+
 // one wavefront per (token, kv head)
 template <typename T>
 __global__ void knorm_kvstore_kernel(const T* __restrict__ k, const T* __restrict__ v, int64_t stride, const T* __restrict__ knorm,
                                      float eps, int G, int d, int dv, int block_size, const int32_t* __restrict__ slots,
+                                     const int64_t* __restrict__ pos, const float* __restrict__ rot_freq, int rot_dims,
                                      T* __restrict__ k_cache, T* __restrict__ v_cache) {
   const int64_t t = blockIdx.x;
   const int g = blockIdx.y, lane = threadIdx.x;
@@ -28,10 +38,19 @@ __global__ void knorm_kvstore_kernel(const T* __restrict__ k, const T* __restric
   float r = 1.f;
   if (knorm) r = rsqrtf(wave_sum(ss) / (float)d + eps);
   T* kc = k_cache + (slot * G + g) * d;
+  const float pf = rot_dims > 0 ? (float)pos[t] : 0.f;
 #pragma unroll
   for (int i = 0; i < MAX_HEAD / 64; ++i) {
     const int c = lane + 64 * i;
-    if (c < d) stf(kc + c, knorm ? kv[i] * r * ldf(knorm + c) : kv[i]);
+    float val = (knorm && c < d) ? kv[i] * r * ldf(knorm + c) : kv[i];
+    // rotation of the pair (2i, 2i+1): the partner sits in the neighbouring lane
+    const float other = __shfl_xor(val, 1, 64);
+    if (c < rot_dims) {
+      float sn, cs;
+      sincosf(pf * rot_freq[c >> 1], &sn, &cs);
+      val = (c & 1) ? val * cs + other * sn : val * cs - other * sn;
+    }
+    if (c < d) stf(kc + c, val);
   }
   const T* vp = v + t * stride + (int64_t)g * dv;
   // values are kept transposed inside a page, [page][G][dv][block]: the attention kernels read a column's consecutive tokens
@@ -47,8 +66,8 @@ __global__ void window_attn_kernel(const T* __restrict__ q, int64_t q_stride, co
                                    const T* __restrict__ gate, int64_t gate_stride, const T* __restrict__ k_cache,
                                    const T* __restrict__ v_cache, const int32_t* __restrict__ block_tables, int64_t bt_stride,
                                    int block_size, const int32_t* __restrict__ cu_q, const int32_t* __restrict__ ctx0,
-                                   const int32_t* __restrict__ tseq, int H, int G, int d, int dv, float scale, int window,
-                                   T* __restrict__ out) {
+                                   const int32_t* __restrict__ tseq, int H, int G, int d, int dv, float scale, int window, int chunk,
+                                   const float* __restrict__ rot_freq, int rot_dims, T* __restrict__ out) {
   __shared__ float qs[MAX_HEAD];
   __shared__ float ps[64];
   __shared__ int64_t slot_s[64];                    // element offset of (token, column 0) in the page-transposed V cache
@@ -72,11 +91,18 @@ __global__ void window_attn_kernel(const T* __restrict__ q, int64_t q_stride, co
 #pragma unroll
     for (int i = 0; i < MAX_HEAD / 64; ++i) {
       const int c = lane + 64 * i;
-      if (c < d) qs[c] = qnorm ? qv[i] * r * ldf(qnorm + c) : qv[i];
+      float val = (qnorm && c < d) ? qv[i] * r * ldf(qnorm + c) : qv[i];
+      const float other = __shfl_xor(val, 1, 64);   // rotation of the pair (2i, 2i+1)
+      if (c < rot_dims) {
+        float sn, cs;
+        sincosf((float)pos * rot_freq[c >> 1], &sn, &cs);
+        val = (c & 1) ? val * cs + other * sn : val * cs - other * sn;
+      }
+      if (c < d) qs[c] = val;
     }
   }
   __syncthreads();
-  const int64_t lo = window > 0 ? (pos - window + 1 > 0 ? pos - window + 1 : 0) : 0;
+  const int64_t lo = vis_lo((int)pos, window, chunk);
   const int32_t* bt = block_tables + (int64_t)s * bt_stride;
   float m = -INFINITY, l = 0.f;
   float acc[MAX_HEAD / 64];
@@ -153,8 +179,8 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(
     const bf16_t* __restrict__ q, int64_t q_stride, const bf16_t* __restrict__ qnorm, float eps, const bf16_t* __restrict__ gate,
     int64_t gate_stride, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int32_t* __restrict__ block_tables, int64_t bt_stride, int block_size, const int32_t* __restrict__ cu_q,
-    const int32_t* __restrict__ ctx0, int nseq, int H, int G, int d, int dv, float scale, int window, int bs_shift,
-    bf16_t* __restrict__ out) {
+    const int32_t* __restrict__ ctx0, int nseq, int H, int G, int d, int dv, float scale, int window, int chunk,
+    const float* __restrict__ rot_freq, int rot_dims, int bs_shift, bf16_t* __restrict__ out) {
   constexpr int QW = 16 * QT;                       // queries per wavefront
   const int lane = threadIdx.x & 63, qi = lane & 15, gq = lane >> 4;
   int tile = blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -204,13 +230,24 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(
 #pragma unroll
     for (int c = 0; c < DK; ++c)
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
+      for (int e = 0; e < 8; e += 2) {
         const int col = c * 32 + gq * 8 + e;
-        const float w = (qnorm && col < d) ? (float)qnorm[col] : 1.f;
-        qb[t][c][e] = (bf16_t)(qv[c][e] * r * w);
+        const float w0 = (qnorm && col < d) ? (float)qnorm[col] : 1.f;
+        const float w1 = (qnorm && col + 1 < d) ? (float)qnorm[col + 1] : 1.f;
+        float a = qv[c][e] * r * w0, b = qv[c][e + 1] * r * w1;
+        if (col < rot_dims) {                        // the pair (2i, 2i+1) turns by pos * freq[i]; both halves are this lane's
+          float sn, cs;
+          sincosf((float)pos[t] * rot_freq[col >> 1], &sn, &cs);
+          const float a2 = a * cs - b * sn;
+          b = b * cs + a * sn;
+          a = a2;
+        }
+        qb[t][c][e] = (bf16_t)a;
+        qb[t][c][e + 1] = (bf16_t)b;
       }
   }
-  const int lo = window > 0 ? (p_first - window + 1 > 0 ? p_first - window + 1 : 0) : 0;
+  const int lo = vis_lo(p_first, window, chunk);
+  const int lo_hi = vis_lo(c0 + tile * QW + QW - 1, window, chunk);      // the tile's last query sees the least far back
   const int32_t* bt = block_tables + (int64_t)s * bt_stride;
   float m[QT], lsum[QT];
   f32x4_t oacc[QT][DVB];
@@ -225,7 +262,7 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(
 
   for (int j0 = lo & ~31; j0 <= p_last; j0 += 64) {
     // every query of the wavefront sees all 64 tokens of the round: no masks (most rounds of a long window)
-    const bool interior = j0 + 63 <= p_first && (window <= 0 || c0 + tile * QW + QW - 1 - j0 < window);
+    const bool interior = j0 + 63 <= p_first && j0 >= lo_hi;
     // ---- S^T for 64 tokens: 4 key blocks, every K fragment feeds all QT tiles
     f32x4_t sacc[QT][4];
 #pragma unroll
@@ -261,7 +298,7 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
             const int j = j0 + (kb >> 1) * 32 + gq * 8 + (kb & 1) * 4 + r;
-            const bool ok = valid_q[t] && j <= pos[t] && (window <= 0 || pos[t] - j < window);
+            const bool ok = valid_q[t] && j <= pos[t] && j >= vis_lo(pos[t], window, chunk);
             okbits |= ok ? (1u << (kb * 4 + r)) : 0u;
           }
       }
@@ -345,8 +382,8 @@ __global__ __launch_bounds__(256) void window_attn_mfma_lds_kernel(
     const bf16_t* __restrict__ q, int64_t q_stride, const bf16_t* __restrict__ qnorm, float eps, const bf16_t* __restrict__ gate,
     int64_t gate_stride, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int32_t* __restrict__ block_tables, int64_t bt_stride, int block_size, const int32_t* __restrict__ cu_q,
-    const int32_t* __restrict__ ctx0, int nseq, int H, int G, int d, int dv, float scale, int window, int bs_shift, int hw,
-    bf16_t* __restrict__ out) {
+    const int32_t* __restrict__ ctx0, int nseq, int H, int G, int d, int dv, float scale, int window, int chunk,
+    const float* __restrict__ rot_freq, int rot_dims, int bs_shift, int hw, bf16_t* __restrict__ out) {
   constexpr int QW = 16 * QT, KP = 32 * DK + 8, VP = 64 + 8, VU = DVB / 2;
   __shared__ __attribute__((aligned(16))) bf16_t Ks[64][KP];
   __shared__ __attribute__((aligned(16))) bf16_t Vs[16 * DVB][VP];
@@ -400,10 +437,20 @@ __global__ __launch_bounds__(256) void window_attn_mfma_lds_kernel(
 #pragma unroll
     for (int c = 0; c < DK; ++c)
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
+      for (int e = 0; e < 8; e += 2) {
         const int col = c * 32 + gq * 8 + e;
-        const float w = (qnorm && col < d) ? (float)qnorm[col] : 1.f;
-        qb[t][c][e] = (bf16_t)(qv[c][e] * r * w);
+        const float w0 = (qnorm && col < d) ? (float)qnorm[col] : 1.f;
+        const float w1 = (qnorm && col + 1 < d) ? (float)qnorm[col + 1] : 1.f;
+        float a = qv[c][e] * r * w0, b = qv[c][e + 1] * r * w1;
+        if (col < rot_dims) {                        // the pair (2i, 2i+1) turns by pos * freq[i]; both halves are this lane's
+          float sn, cs;
+          sincosf((float)pos[t] * rot_freq[col >> 1], &sn, &cs);
+          const float a2 = a * cs - b * sn;
+          b = b * cs + a * sn;
+          a = a2;
+        }
+        qb[t][c][e] = (bf16_t)a;
+        qb[t][c][e + 1] = (bf16_t)b;
       }
   }
   float m[QT], lsum[QT];
@@ -451,7 +498,8 @@ __global__ __launch_bounds__(256) void window_attn_mfma_lds_kernel(
       }
     }
   };
-  const int lo = window > 0 ? (b_first - window + 1 > 0 ? b_first - window + 1 : 0) : 0;
+  const int lo = vis_lo(b_first, window, chunk);
+  const int lo_first = vis_lo(p_first, window, chunk), lo_hi = vis_lo(p_hi, window, chunk);
   int j0 = lo & ~31;
   lookup(j0);
   fetch(j0);
@@ -474,8 +522,8 @@ __global__ __launch_bounds__(256) void window_attn_mfma_lds_kernel(
       lookup(j0 + 128);
     }
     // a wavefront whose queries all lie before the round's tokens (or beyond the portion) has nothing to add
-    if (j0 > p_hi || rel0 >= len || (window > 0 && j0 + 63 < p_first - window + 1)) continue;
-    const bool interior = j0 + 63 <= p_first && (window <= 0 || p_hi - j0 < window);
+    if (j0 > p_hi || rel0 >= len || j0 + 63 < lo_first) continue;
+    const bool interior = j0 + 63 <= p_first && j0 >= lo_hi;
     f32x4_t sacc[QT][4];
 #pragma unroll
     for (int kb = 0; kb < 4; ++kb) {
@@ -501,7 +549,7 @@ __global__ __launch_bounds__(256) void window_attn_mfma_lds_kernel(
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
             const int j = j0 + (kb >> 1) * 32 + gq * 8 + (kb & 1) * 4 + r;
-            const bool ok = valid_q[t] && j <= pos[t] && (window <= 0 || pos[t] - j < window);
+            const bool ok = valid_q[t] && j <= pos[t] && j >= vis_lo(pos[t], window, chunk);
             okbits |= ok ? (1u << (kb * 4 + r)) : 0u;
           }
       }
@@ -565,7 +613,7 @@ template <int DK, int DVB, int QT>
 void launch_mfma_qt(const void* q, int64_t q_stride, const void* qnorm, float eps, const void* gate, int64_t gate_stride,
                     const void* k_cache, const void* v_cache, const int32_t* block_tables, int64_t bt_stride, int block_size,
                     const int32_t* cu_q, const int32_t* ctx0, int nseq, int64_t n, int H, int G, int d, int dv, float scale, int window,
-                    void* out, hipStream_t stream) {
+                    int chunk, const float* rot_freq, int rot_dims, void* out, hipStream_t stream) {
   int bs_shift = -1;
   for (int b = 0; b < 31; ++b)
     if ((1 << b) == block_size) bs_shift = b;
@@ -576,15 +624,16 @@ void launch_mfma_qt(const void* q, int64_t q_stride, const void* qnorm, float ep
       const int64_t btiles = n / bq + nseq;         // an upper bound: every portion may end with a partial tile
       window_attn_mfma_lds_kernel<DK, DVB, QT><<<dim3((unsigned)btiles, (unsigned)(G * (hpg / hw))), dim3(256), 0, stream>>>(
           (const bf16_t*)q, q_stride, (const bf16_t*)qnorm, eps, (const bf16_t*)gate, gate_stride, (const bf16_t*)k_cache,
-          (const bf16_t*)v_cache, block_tables, bt_stride, block_size, cu_q, ctx0, nseq, H, G, d, dv, scale, window, bs_shift, hw,
-          (bf16_t*)out);
+          (const bf16_t*)v_cache, block_tables, bt_stride, block_size, cu_q, ctx0, nseq, H, G, d, dv, scale, window, chunk, rot_freq,
+          rot_dims, bs_shift, hw, (bf16_t*)out);
       return;
     }
   }
   const int64_t tiles = n / (16 * QT) + nseq;       // an upper bound: every portion may end with a partial tile
   window_attn_mfma_kernel<DK, DVB, QT><<<dim3((unsigned)((tiles + 3) / 4), H), dim3(256), 0, stream>>>(
       (const bf16_t*)q, q_stride, (const bf16_t*)qnorm, eps, (const bf16_t*)gate, gate_stride, (const bf16_t*)k_cache,
-      (const bf16_t*)v_cache, block_tables, bt_stride, block_size, cu_q, ctx0, nseq, H, G, d, dv, scale, window, bs_shift, (bf16_t*)out);
+      (const bf16_t*)v_cache, block_tables, bt_stride, block_size, cu_q, ctx0, nseq, H, G, d, dv, scale, window, chunk, rot_freq, rot_dims,
+      bs_shift, (bf16_t*)out);
 }
 
 // Long portions (prefill) put two tiles of 16 queries on a wavefront: half the K / V bytes through the vector cache per
@@ -593,13 +642,13 @@ template <int DK, int DVB>
 void launch_mfma(const void* q, int64_t q_stride, const void* qnorm, float eps, const void* gate, int64_t gate_stride,
                  const void* k_cache, const void* v_cache, const int32_t* block_tables, int64_t bt_stride, int block_size,
                  const int32_t* cu_q, const int32_t* ctx0, int nseq, int64_t n, int H, int G, int d, int dv, float scale, int window,
-                 void* out, hipStream_t stream) {
+                 int chunk, const float* rot_freq, int rot_dims, void* out, hipStream_t stream) {
   if (n >= 32ll * nseq)
     launch_mfma_qt<DK, DVB, 2>(q, q_stride, qnorm, eps, gate, gate_stride, k_cache, v_cache, block_tables, bt_stride, block_size, cu_q,
-                               ctx0, nseq, n, H, G, d, dv, scale, window, out, stream);
+                               ctx0, nseq, n, H, G, d, dv, scale, window, chunk, rot_freq, rot_dims, out, stream);
   else
     launch_mfma_qt<DK, DVB, 1>(q, q_stride, qnorm, eps, gate, gate_stride, k_cache, v_cache, block_tables, bt_stride, block_size, cu_q,
-                               ctx0, nseq, n, H, G, d, dv, scale, window, out, stream);
+                               ctx0, nseq, n, H, G, d, dv, scale, window, chunk, rot_freq, rot_dims, out, stream);
 }
 }  // namespace
 
@@ -611,21 +660,29 @@ extern "C" void nvs_window_attn_force_scalar(int on) {
 }
 
 extern "C" int nvs_knorm_kvstore(const void* k, const void* v, int64_t stride, int dtype, const void* knorm, float eps, int G, int d,
-                                 int dv, int block_size, const int32_t* slots, int64_t n, void* k_cache, void* v_cache, void* stream) {
+                                 int dv, int block_size, const int32_t* slots, const int64_t* pos, const float* rot_freq, int rot_dims,
+                                 int64_t n, void* k_cache, void* v_cache, void* stream) {
   NVS_REQUIRE(k && v && slots && k_cache && v_cache, "nvs_knorm_kvstore: null argument");
+  NVS_REQUIRE(rot_dims >= 0 && rot_dims % 2 == 0 && rot_dims <= d && (rot_dims == 0 || (pos && rot_freq)),
+              "nvs_knorm_kvstore: rotation of %d of %d dimensions", rot_dims, d);
   NVS_REQUIRE(G > 0 && G <= 65535 && d > 0 && d <= MAX_HEAD && dv > 0 && dv <= MAX_HEAD && n >= 0 && block_size > 0,
               "nvs_knorm_kvstore: G %d d %d dv %d", G, d, dv);
   if (n == 0) return NVS_OK;
   NVS_DISPATCH(dtype, knorm_kvstore_kernel<T><<<dim3((unsigned)n, G), dim3(64), 0, (hipStream_t)stream>>>(
-                          (const T*)k, (const T*)v, stride, (const T*)knorm, eps, G, d, dv, block_size, slots, (T*)k_cache, (T*)v_cache));
+                          (const T*)k, (const T*)v, stride, (const T*)knorm, eps, G, d, dv, block_size, slots, pos, rot_freq, rot_dims, (T*)k_cache,
+                          (T*)v_cache));
   return nvs_check_launch("nvs_knorm_kvstore");
 }
 
 extern "C" int nvs_window_attn(const void* q, int64_t q_stride, const void* qnorm, float eps, const void* gate, int64_t gate_stride,
                                int dtype, const void* k_cache, const void* v_cache, const int32_t* block_tables, int64_t bt_stride,
                                int block_size, const int32_t* cu_q, const int32_t* ctx0, const int32_t* tseq, int nseq, int64_t n, int H,
-                               int G, int d, int dv, float scale, int window, void* out, void* stream) {
+                               int G, int d, int dv, float scale, int window, int chunk, const float* rot_freq, int rot_dims, void* out,
+                               void* stream) {
   NVS_REQUIRE(q && k_cache && v_cache && block_tables && cu_q && ctx0 && tseq && out, "nvs_window_attn: null argument");
+  NVS_REQUIRE(!(window > 0 && chunk > 0), "nvs_window_attn: a window (%d) and blocks (%d) together", window, chunk);
+  NVS_REQUIRE(rot_dims >= 0 && rot_dims % 2 == 0 && rot_dims <= d && (rot_dims == 0 || rot_freq),
+              "nvs_window_attn: rotation of %d of %d dimensions", rot_dims, d);
   NVS_REQUIRE(H > 0 && H <= 65535 && G > 0 && H % G == 0 && d > 0 && d <= MAX_HEAD && dv > 0 && dv <= MAX_HEAD && block_size > 0 && n >= 0,
               "nvs_window_attn: H %d G %d d %d dv %d block %d", H, G, d, dv, block_size);
   if (n == 0 || nseq == 0) return NVS_OK;
@@ -634,7 +691,7 @@ extern "C" int nvs_window_attn(const void* q, int64_t q_stride, const void* qnor
 #define NVS_MFMA_CASE(DK, DVB)                                                                                                  \
   if (dk == DK && dvb == DVB)                                                                                                   \
     launch_mfma<DK, DVB>(q, q_stride, qnorm, eps, gate, gate_stride, k_cache, v_cache, block_tables, bt_stride, block_size, cu_q, \
-                         ctx0, nseq, n, H, G, d, dv, scale, window, out, (hipStream_t)stream);
+                         ctx0, nseq, n, H, G, d, dv, scale, window, chunk, rot_freq, rot_dims, out, (hipStream_t)stream);
     NVS_MFMA_CASE(2, 4) NVS_MFMA_CASE(2, 8) NVS_MFMA_CASE(2, 16) NVS_MFMA_CASE(4, 4) NVS_MFMA_CASE(4, 8) NVS_MFMA_CASE(4, 16)
     NVS_MFMA_CASE(8, 4) NVS_MFMA_CASE(8, 8) NVS_MFMA_CASE(8, 16)
 #undef NVS_MFMA_CASE
@@ -642,6 +699,6 @@ extern "C" int nvs_window_attn(const void* q, int64_t q_stride, const void* qnor
   }
   NVS_DISPATCH(dtype, window_attn_kernel<T><<<dim3((unsigned)n, H), dim3(64), 0, (hipStream_t)stream>>>(
                           (const T*)q, q_stride, (const T*)qnorm, eps, (const T*)gate, gate_stride, (const T*)k_cache, (const T*)v_cache,
-                          block_tables, bt_stride, block_size, cu_q, ctx0, tseq, H, G, d, dv, scale, window, (T*)out));
+                          block_tables, bt_stride, block_size, cu_q, ctx0, tseq, H, G, d, dv, scale, window, chunk, rot_freq, rot_dims, (T*)out));
   return nvs_check_launch("nvs_window_attn");
 }

@@ -20,7 +20,7 @@ int nvs_check_launch(const char* what) {
   }
   return NVS_OK;
 }
-extern "C" int nvs_abi_version(void) { return 2; }   // 2: segmented SSD scan (workspace, longest portion)
+extern "C" int nvs_abi_version(void) { return 3; }   // 3: block masks and rotation in attention, pre-norm kernels, decay scan, routed experts
 extern "C" const char* nvs_last_error(void) { return g_err; }
 
 namespace {
@@ -36,7 +36,7 @@ __global__ void embed_sinusoid_kernel(const T* __restrict__ table, const int64_t
     // base^(-2i/width) in 32-bit; the angle is the product of two 32-bit numbers
     const float inv = exp2f(-(2.f * (float)i / (float)width) * log2_base);
     const float ang = p * inv;
-    const float pe = (c & 1) ? cosf(ang) : sinf(ang);
+    const float pe = log2_base > 0.f ? ((c & 1) ? cosf(ang) : sinf(ang)) : 0.f;      // (no base: no sinusoid)
     const float v = ldf(table + id * width + c) * scale + pe;
     x[t * width + c] = v;
     if (xh) stf(xh + t * width + c, v);
@@ -112,16 +112,43 @@ __global__ void xielu_kernel(const T* __restrict__ in, const T* __restrict__ pq,
   }
 }
 
+// Input-side ("pre") norm on the 32-bit residual: x[t] += a[t] + b[t] first (either may be absent), then every one of
+// `groups` equal parts of the row is divided by its own root mean square and the row is multiplied by w. One workgroup per
+// row, one wavefront per group at a time. With `rows` the kernel only reads: out[r] = norm(x[rows[r]]).
+template <typename T>
+__global__ void add_group_norm_kernel(float* __restrict__ x, const T* __restrict__ a, const float* __restrict__ b,
+                                      const int32_t* __restrict__ rows, const T* __restrict__ w, int width, int groups, float eps,
+                                      T* __restrict__ out) {
+  const int64_t r = blockIdx.x;
+  const int64_t t = rows ? (int64_t)rows[r] : r;
+  const int gsz = width / groups, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  float* xr = x + t * width;
+  for (int g = wave; g < groups; g += nw) {
+    const int c0 = g * gsz;
+    float ss = 0.f;
+    for (int c = lane; c < gsz; c += 64) {
+      float v = xr[c0 + c];
+      if (a) v += ldf(a + t * width + c0 + c);
+      if (b) v += b[t * width + c0 + c];
+      if (a || b) xr[c0 + c] = v;
+      ss += v * v;
+    }
+    if (!out) continue;
+    const float k = 1.f / sqrtf(wave_sum(ss) / (float)gsz + eps);
+    for (int c = lane; c < gsz; c += 64) stf(out + r * width + c0 + c, xr[c0 + c] * k * ldf(w + c0 + c));   // (this lane wrote xr[c0 + c])
+  }
+}
+
 int threads_for(int width) { return width >= 1024 ? 256 : (width >= 256 ? 128 : 64); }
 
 }  // namespace
 
 extern "C" int nvs_embed_sinusoid(const void* table, int dtype, const int64_t* ids, const int64_t* pos, int64_t n, int width,
                                   float scale, float base, float* x, void* xh, void* stream) {
-  NVS_REQUIRE(table && ids && pos && x && n >= 0 && width > 0 && base > 1.f, "nvs_embed_sinusoid: bad argument");
+  NVS_REQUIRE(table && ids && pos && x && n >= 0 && width > 0 && (base > 1.f || base == 0.f), "nvs_embed_sinusoid: bad argument");
   if (n == 0) return NVS_OK;
   NVS_DISPATCH(dtype, embed_sinusoid_kernel<T><<<dim3((unsigned)n), dim3(threads_for(width)), 0, (hipStream_t)stream>>>(
-                          (const T*)table, ids, pos, width, scale, log2f(base), x, (T*)xh));
+                          (const T*)table, ids, pos, width, scale, base > 1.f ? log2f(base) : 0.f, x, (T*)xh));
   return nvs_check_launch("nvs_embed_sinusoid");
 }
 
@@ -151,4 +178,16 @@ extern "C" int nvs_xielu(const void* in, const void* pq, float beta, int dtype, 
   NVS_DISPATCH(dtype, xielu_kernel<T><<<dim3((unsigned)(blocks > 65536 ? 65536 : blocks)), dim3(256), 0, (hipStream_t)stream>>>(
                           (const T*)in, (const T*)pq, beta, numel, (T*)out));
   return nvs_check_launch("nvs_xielu");
+}
+
+extern "C" int nvs_add_group_norm(float* x, const void* a, const float* b, const int32_t* rows, int64_t nrows, const void* w, int dtype,
+                                  int width, int groups, float eps, void* out, void* stream) {
+  NVS_REQUIRE(x && nrows >= 0 && width > 0 && groups > 0 && width % groups == 0 && (!out || w), "nvs_add_group_norm: width %d groups %d",
+              width, groups);
+  NVS_REQUIRE(!rows || (!a && !b), "nvs_add_group_norm: selected rows are only read");
+  if (nrows == 0) return NVS_OK;
+  const int threads = 64 * (groups < 4 ? groups : 4);      // a wavefront per group, four groups at a time
+  NVS_DISPATCH(dtype, add_group_norm_kernel<T><<<dim3((unsigned)nrows), dim3(threads), 0, (hipStream_t)stream>>>(
+                          x, (const T*)a, b, rows, (const T*)w, width, groups, eps, (T*)out));
+  return nvs_check_launch("nvs_add_group_norm");
 }

@@ -161,8 +161,13 @@ constexpr int SSD_R = 16;      // state entries per thread
 constexpr int SSD_TB = 16;     // tokens per LDS round
 constexpr int SSD_SB = 8;      // tokens whose cross-lane sums are taken together
 
-template <typename T, int PP, int MODE>     // PP head-size entries per thread: the B / C values read from LDS serve PP state rows
+// FORM 0: the state-space-duality recurrence as described above. FORM 1: the decaying outer-product recurrence of linear
+// ("lightning") attention, S <- decay_h S + k v^T, o = S^T q — the same walk with x = v, B = k, C = q, a step size of one, a
+// decay that is a per-head constant (`decay`, 32-bit) and no skip term; v | k | q are read from the projection output itself
+// (columns x_col / b_col / c_col + the head's offset, `dtype`) and SiLU is applied as they are staged.
+template <typename T, int PP, int MODE, int FORM = 0>     // PP head-size entries per thread: the B / C values read from LDS serve PP state rows
 __global__ __launch_bounds__(PP == 4 ? 256 : (PP == 2 ? 512 : 1024)) void ssd_scan_kernel(const float* __restrict__ xbc, const T* __restrict__ proj, int64_t proj_stride, int64_t dt_col,
+                                int64_t x_col, int64_t b_col, int64_t c_col, const float* __restrict__ decay,
                                 const T* __restrict__ dt_bias, const T* __restrict__ A_log, const T* __restrict__ Dp, int heads,
                                 int P, int N, int G, int NG, int TB, const int32_t* __restrict__ cu_q,
                                 const int32_t* __restrict__ ctx0, const int32_t* __restrict__ slot, float* __restrict__ S,
@@ -188,7 +193,12 @@ __global__ __launch_bounds__(PP == 4 ? 256 : (PP == 2 ? 512 : 1024)) void ssd_sc
   const int NP = NG * SSD_R, P4 = (P + 3) & ~3, per = P4 + 2 * NP + 4;    // every part starts 16-byte aligned
   const int inner = heads * P, grp = h / (heads / G);
   const int64_t row = inner + 2 * G * N;
-  const float A = -expf(ldf(A_log + h)), Dh = ldf(Dp + h), dtb = ldf(dt_bias + h);
+  float A = 0.f, Dh = 0.f, dtb = 0.f, fixed_decay = 1.f;
+  if (FORM == 0) {
+    A = -expf(ldf(A_log + h)), Dh = ldf(Dp + h), dtb = ldf(dt_bias + h);
+  } else {
+    fixed_decay = decay[h];
+  }
   float* Sh = S + (((int64_t)slot[s] * heads + h) * P + p) * N + g * SSD_R;
   float st[PP][SSD_R];
   const bool fresh = ctx0[s] == 0;
@@ -246,6 +256,9 @@ __global__ __launch_bounds__(PP == 4 ? 256 : (PP == 2 ? 512 : 1024)) void ssd_sc
   float* yh = y + h * P + p;
   const float* Bg = xbc + inner + grp * N;
   const float* Cg = Bg + G * N;
+  const T* xh1 = proj + x_col + h * P;              // FORM 1: the three operands inside the projection output
+  const T* Bg1 = proj + b_col + grp * N;
+  const T* Cg1 = proj + c_col + grp * N;
   for (int64_t tb = q0; tb < q1; tb += TB) {
     const int cnt = (int)((q1 - tb) < TB ? (q1 - tb) : TB);
     __syncthreads();                                // the previous round's readers are done
@@ -254,13 +267,14 @@ __global__ __launch_bounds__(PP == 4 ? 256 : (PP == 2 ? 512 : 1024)) void ssd_sc
     // independent and in flight together, and for a fixed token neighbouring threads read neighbouring addresses
     for (int c = tid; c < per; c += nthreads) {
       const float* src = nullptr;                   // a 32-bit source with row stride `row`
+      const T* src1 = nullptr;                      // FORM 1: a source in the projection output, SiLU applied here
       int kind = 0;                                 // 0: padding (zero), 1: x / B / C, 2: step size, 3: decay
       if (c < P) {
-        src = xh + c, kind = 1;
+        src = xh + c, src1 = xh1 + c, kind = 1;
       } else if (c >= P4 && c < P4 + NP) {
-        if (c - P4 < N) src = Bg + (c - P4), kind = 1;
+        if (c - P4 < N) src = Bg + (c - P4), src1 = Bg1 + (c - P4), kind = 1;
       } else if (c >= P4 + NP && c < P4 + 2 * NP) {
-        if (c - P4 - NP < N) src = Cg + (c - P4 - NP), kind = 1;
+        if (c - P4 - NP < N) src = Cg + (c - P4 - NP), src1 = Cg1 + (c - P4 - NP), kind = 1;
       } else if (c == P4 + 2 * NP) {
         kind = 2;
       } else if (c == P4 + 2 * NP + 1) {
@@ -271,17 +285,27 @@ __global__ __launch_bounds__(PP == 4 ? 256 : (PP == 2 ? 512 : 1024)) void ssd_sc
       for (int k = 0; k < SSD_TB; ++k) {
         v[k] = 0.f;
         if (k < cnt) {
-          if (kind == 1) v[k] = src[(tb + k) * row];
-          if (kind >= 2) v[k] = ldf(proj + (tb + k) * proj_stride + dt_col + h);
+          if (FORM == 0) {
+            if (kind == 1) v[k] = src[(tb + k) * row];
+            if (kind >= 2) v[k] = ldf(proj + (tb + k) * proj_stride + dt_col + h);
+          } else {
+            if (kind == 1) v[k] = ldf(src1 + (tb + k) * proj_stride);
+          }
         }
       }
 #pragma unroll
       for (int k = 0; k < SSD_TB; ++k) {
         if (k < cnt) {
           float w = v[k];
-          if (kind >= 2) {
-            w = softplusf_(w + dtb);
-            if (kind == 3) w = expf(A * w);
+          if (FORM == 0) {
+            if (kind >= 2) {
+              w = softplusf_(w + dtb);
+              if (kind == 3) w = expf(A * w);
+            }
+          } else {
+            if (kind == 1) w = siluf_(w);
+            if (kind == 2) w = 1.f;
+            if (kind == 3) w = fixed_decay;
           }
           lds[k * per + c] = w;
         }
@@ -365,11 +389,23 @@ __global__ __launch_bounds__(PP == 4 ? 256 : (PP == 2 ? 512 : 1024)) void ssd_sc
 // one workgroup per (token, group)
 template <typename T>
 __global__ void gated_group_norm_kernel(const float* __restrict__ y, const T* __restrict__ z, int64_t z_stride,
-                                        const T* __restrict__ w, int inner, int groups, float eps, T* __restrict__ out) {
+                                        const T* __restrict__ w, int inner, int groups, float eps, int order, T* __restrict__ out) {
   __shared__ float red[16];
   const int64_t t = blockIdx.y;
   const int gsz = inner / groups, c0 = blockIdx.x * gsz;
   float ss = 0.f;
+  if (order == 1) {                                 // norm first, then a sigmoid gate
+    for (int c = threadIdx.x; c < gsz; c += blockDim.x) {
+      const float v = y[t * inner + c0 + c];
+      ss += v * v;
+    }
+    const float r = 1.f / sqrtf(block_sum(ss, red) / (float)gsz + eps);
+    for (int c = threadIdx.x; c < gsz; c += blockDim.x) {
+      const float gz = ldf(z + t * z_stride + c0 + c);
+      stf(out + t * inner + c0 + c, y[t * inner + c0 + c] * r * ldf(w + c0 + c) * (1.f / (1.f + expf(-gz))));
+    }
+    return;
+  }
   for (int c = threadIdx.x; c < gsz; c += blockDim.x) {
     const float v = y[t * inner + c0 + c] * siluf_(ldf(z + t * z_stride + c0 + c));
     ss += v * v;
@@ -460,13 +496,13 @@ extern "C" int64_t nvs_ssd_scan_workspace(int heads, int P, int N, int nseq, int
   return seg_len ? (int64_t)nseq * heads * (nseg + 1) * ((int64_t)P * N + 1) : 0;
 }
 
-extern "C" int nvs_ssd_scan(const float* xbc, const void* proj, int64_t proj_stride, int64_t dt_col, int dtype, const void* dt_bias,
-                            const void* A_log, const void* D, int heads, int P, int N, int G, const int32_t* cu_q, const int32_t* ctx0,
-                            const int32_t* slot, int nseq, int64_t n, int64_t max_q, float* S, float* y, float* ws, int64_t ws_floats,
-                            void* stream) {
-  NVS_REQUIRE(xbc && proj && dt_bias && A_log && D && cu_q && ctx0 && slot && S && y, "nvs_ssd_scan: null argument");
+// both forms of the scan: argument checks that they share, the plan, the launches
+static int ssd_launch(int form, const char* who, const float* xbc, const void* proj, int64_t proj_stride, int64_t dt_col, int64_t x_col,
+                      int64_t b_col, int64_t c_col, const float* decay, int dtype, const void* dt_bias, const void* A_log, const void* D,
+                      int heads, int P, int N, int G, const int32_t* cu_q, const int32_t* ctx0, const int32_t* slot, int nseq, int64_t n,
+                      int64_t max_q, float* S, float* y, float* ws, int64_t ws_floats, void* stream) {
   NVS_REQUIRE(heads > 0 && G > 0 && heads % G == 0 && P > 0 && P <= 256 && N > 0 && nseq >= 0 && nseq <= 65535,
-              "nvs_ssd_scan: heads %d groups %d head size %d state %d", heads, G, P, N);
+              "%s: heads %d groups %d head size %d state %d", who, heads, G, P, N);
   if (n == 0 || nseq == 0) return NVS_OK;
   int ng = 1;
   while (ng * SSD_R < N) ng <<= 1;                  // a power of two: the threads of one p reduce by lane shuffles
@@ -478,42 +514,71 @@ extern "C" int nvs_ssd_scan(const float* xbc, const void* proj, int64_t proj_str
   static const int forced = getenv("NVS_SSD_PP") ? atoi(getenv("NVS_SSD_PP")) : 0;
   int pp = forced ? forced : 2;
   while (pp > 1 && (P % pp != 0 || (P / pp) * ng0 > (pp == 4 ? 256 : 512))) pp >>= 1;
-  NVS_REQUIRE(ng <= 64 && (int64_t)(P / pp) * ng <= 1024, "nvs_ssd_scan: state %d x head size %d exceeds one workgroup's registers", N, P);
+  NVS_REQUIRE(ng <= 64 && (int64_t)(P / pp) * ng <= 1024, "%s: state %d x head size %d exceeds one workgroup's registers", who, N, P);
   const int threads = (P / pp) * ng, per = ((P + 3) & ~3) + 2 * ng * SSD_R + 4;
   const int tb = SSD_TB;                            // tokens per LDS round
   const size_t lds = (size_t)tb * per * sizeof(float);
   int seg_len = 0, nseg = 1;
   if (ws) ssd_plan(heads, nseq, max_q > 0 ? max_q : n, &seg_len, &nseg);
   NVS_REQUIRE(!seg_len || ws_floats >= nvs_ssd_scan_workspace(heads, P, N, nseq, max_q > 0 ? max_q : n),
-              "nvs_ssd_scan: workspace of %lld floats is too small", (long long)ws_floats);
+              "%s: workspace of %lld floats is too small", who, (long long)ws_floats);
   const dim3 grid(heads, (unsigned)nseq, seg_len ? nseg : 1);
-#define NVS_SSD_LAUNCH(PPV, MODE)                                                                                                   \
-  NVS_DISPATCH(dtype, ssd_scan_kernel<T, PPV, MODE><<<grid, dim3(threads), lds, (hipStream_t)stream>>>(                              \
-                          xbc, (const T*)proj, proj_stride, dt_col, (const T*)dt_bias, (const T*)A_log, (const T*)D, heads, P, N, G, ng, \
-                          tb, cu_q, ctx0, slot, S, y, seg_len, nseg, ws))
-#define NVS_SSD_PASSES(PPV)   \
-  if (seg_len) {              \
-    NVS_SSD_LAUNCH(PPV, 1);   \
-    NVS_SSD_LAUNCH(PPV, 2);   \
-  } else {                    \
-    NVS_SSD_LAUNCH(PPV, 0);   \
+#define NVS_SSD_LAUNCH(PPV, MODE, FORM)                                                                                             \
+  NVS_DISPATCH(dtype, ssd_scan_kernel<T, PPV, MODE, FORM><<<grid, dim3(threads), lds, (hipStream_t)stream>>>(                        \
+                          xbc, (const T*)proj, proj_stride, dt_col, x_col, b_col, c_col, decay, (const T*)dt_bias, (const T*)A_log,   \
+                          (const T*)D, heads, P, N, G, ng, tb, cu_q, ctx0, slot, S, y, seg_len, nseg, ws))
+#define NVS_SSD_PASSES(PPV, FORM)   \
+  if (seg_len) {                    \
+    NVS_SSD_LAUNCH(PPV, 1, FORM);   \
+    NVS_SSD_LAUNCH(PPV, 2, FORM);   \
+  } else {                          \
+    NVS_SSD_LAUNCH(PPV, 0, FORM);   \
+  }
+#define NVS_SSD_FORMS(PPV)   \
+  if (form == 0) {           \
+    NVS_SSD_PASSES(PPV, 0)   \
+  } else {                   \
+    NVS_SSD_PASSES(PPV, 1)   \
   }
   if (pp == 2) {
-    NVS_SSD_PASSES(2)
+    NVS_SSD_FORMS(2)
   } else if (pp == 4) {
-    NVS_SSD_PASSES(4)
+    NVS_SSD_FORMS(4)
   } else {
-    NVS_SSD_PASSES(1)
+    NVS_SSD_FORMS(1)
   }
+#undef NVS_SSD_FORMS
 #undef NVS_SSD_PASSES
 #undef NVS_SSD_LAUNCH
-  return nvs_check_launch("nvs_ssd_scan");
+  return nvs_check_launch(who);
+}
+
+extern "C" int nvs_ssd_scan(const float* xbc, const void* proj, int64_t proj_stride, int64_t dt_col, int dtype, const void* dt_bias,
+                            const void* A_log, const void* D, int heads, int P, int N, int G, const int32_t* cu_q, const int32_t* ctx0,
+                            const int32_t* slot, int nseq, int64_t n, int64_t max_q, float* S, float* y, float* ws, int64_t ws_floats,
+                            void* stream) {
+  NVS_REQUIRE(xbc && proj && dt_bias && A_log && D && cu_q && ctx0 && slot && S && y, "nvs_ssd_scan: null argument");
+  return ssd_launch(0, "nvs_ssd_scan", xbc, proj, proj_stride, dt_col, 0, 0, 0, nullptr, dtype, dt_bias, A_log, D, heads, P, N, G, cu_q,
+                    ctx0, slot, nseq, n, max_q, S, y, ws, ws_floats, stream);
+}
+
+extern "C" int nvs_decay_scan(const void* proj, int64_t proj_stride, int64_t v_col, int64_t k_col, int64_t q_col, int dtype,
+                              const float* decay, int heads, int dk, int dv, const int32_t* cu_q, const int32_t* ctx0,
+                              const int32_t* slot, int nseq, int64_t n, int64_t max_q, float* S, float* y, float* ws, int64_t ws_floats,
+                              void* stream) {
+  NVS_REQUIRE(proj && decay && cu_q && ctx0 && slot && S && y, "nvs_decay_scan: null argument");
+  NVS_REQUIRE(v_col >= 0 && k_col >= 0 && q_col >= 0 && v_col + (int64_t)heads * dv <= proj_stride &&
+                  k_col + (int64_t)heads * dk <= proj_stride && q_col + (int64_t)heads * dk <= proj_stride,
+              "nvs_decay_scan: columns beyond the row stride %lld", (long long)proj_stride);
+  return ssd_launch(1, "nvs_decay_scan", nullptr, proj, proj_stride, 0, v_col, k_col, q_col, decay, dtype, nullptr, nullptr, nullptr, heads,
+                    dv, dk, heads, cu_q, ctx0, slot, nseq, n, max_q, S, y, ws, ws_floats, stream);
 }
 
 extern "C" int nvs_gated_group_norm(const float* y, const void* z, int64_t z_stride, int dtype, const void* w, int inner, int groups,
-                                    float eps, int64_t n, void* out, void* stream) {
-  NVS_REQUIRE(y && z && w && out && inner > 0 && groups > 0 && inner % groups == 0 && z_stride >= inner && n >= 0,
-              "nvs_gated_group_norm: inner %d groups %d", inner, groups);
+                                    float eps, int order, int64_t n, void* out, void* stream) {
+  NVS_REQUIRE(y && z && w && out && inner > 0 && groups > 0 && inner % groups == 0 && z_stride >= inner && n >= 0 &&
+                  (order == 0 || order == 1),
+              "nvs_gated_group_norm: inner %d groups %d order %d", inner, groups, order);
   if (n == 0) return NVS_OK;
   NVS_REQUIRE(n <= 65535ll * 65535ll, "nvs_gated_group_norm: step too large");
   const int gsz = inner / groups;
@@ -521,7 +586,7 @@ extern "C" int nvs_gated_group_norm(const float* y, const void* z, int64_t z_str
   for (int64_t t0 = 0; t0 < n; t0 += 65535) {
     const int64_t cnt = n - t0 < 65535 ? n - t0 : 65535;
     NVS_DISPATCH(dtype, gated_group_norm_kernel<T><<<dim3(groups, (unsigned)cnt), block, 0, (hipStream_t)stream>>>(
-                            y + t0 * inner, (const T*)z + t0 * z_stride, z_stride, (const T*)w, inner, groups, eps, (T*)out + t0 * inner));
+                            y + t0 * inner, (const T*)z + t0 * z_stride, z_stride, (const T*)w, inner, groups, eps, order, (T*)out + t0 * inner));
   }
   return nvs_check_launch("nvs_gated_group_norm");
 }

@@ -1,12 +1,19 @@
 """Sequence mixers and feed-forwards beyond full attention, as layers any model of the package can compose:
 
-  WindowAttention     paged softmax attention with a sliding window, any query / value head size, optional per-head
-                      q/k RMS norm, optional sigmoid output gate, no rotation (positions do not enter the scores)
+  WindowAttention     paged softmax attention with a local mask (a sliding window, or blocks of positions, or none), any
+                      query / value head size, optional per-head q/k RMS norm, optional rotation of the leading dimensions
+                      in interleaved pairs, optional sigmoid output gate
+  AttentionMixer      fused biased q | k | v projection -> WindowAttention -> out projection
+  LightningMixer      linear attention as a decaying outer-product recurrence (per-head constant decay), SiLU on q / k / v,
+                      RMS norm over the heads together, sigmoid gate
   SSDMixer            state-space-duality (Mamba-2 style) mixer: stateful causal convolution + SiLU, the recurrence in
                       32-bit, gate-then-group-norm
   RGLRUMixer          recurrent block with a real-gated linear recurrent unit (block-diagonal gates)
   ParallelMixer       two mixers on the same input; the caller averages their RMS-normed outputs
   XIELUFeedForward    up -> xIELU -> down
+  ClampedGLU          [gate | up] -> min(g, limit) sigmoid(alpha g) (clamp(u) + 1) -> down
+  RoutedExperts       mixture of gated experts: softmax router with a choice-only correction, choice limited to the best
+                      groups of experts, pass-through experts, optional shared expert with a sigmoid gate per token
 
 Every constant a design may change is a constructor argument. Matrix products are the vendor library's (F.linear /
 baddbmm); everything else is a kernel of libnvl_seq.so (ops_seq). Layers read the step's packed-portion description from
@@ -41,11 +48,19 @@ class WindowAttention(nn.Module):
     """Consumes q | k | v | gate column ranges of the owner's fused projection output."""
 
     def __init__(self, heads: int, kv_heads: int, dim: int, vdim: int, scale: float, window: int, eps: float,
-                 qk_norm: bool = True, block_size: int = 256):
+                 qk_norm: bool = True, block_size: int = 256, chunk: int = 0, rot_dims: int = 0, rot_base: float = 10000.0):
+        """window > 0: the last `window` positions are visible; chunk > 0: the positions of the query's own block of `chunk`
+        (counted from the start of the sequence); neither: all earlier positions. rot_dims > 0: entries (2i, 2i+1),
+        i < rot_dims / 2, of every query and key head turn by position * rot_base^(-2i / rot_dims)."""
         super().__init__()
-        assert heads % kv_heads == 0 and dim <= 256 and vdim <= 256
+        assert heads % kv_heads == 0 and dim <= 256 and vdim <= 256 and not (window > 0 and chunk > 0)
+        assert rot_dims % 2 == 0 and 0 <= rot_dims <= dim
         self.H, self.G, self.d, self.dv = heads, kv_heads, dim, vdim
         self.scale, self.window, self.eps, self.block_size = float(scale), int(window), eps, block_size
+        self.chunk = int(chunk)
+        # frequencies in double precision on the host, rounded once; angles are position * frequency in 32-bit
+        self.register_buffer("rot_freq", torch.tensor([float(rot_base) ** (-2.0 * i / rot_dims) for i in range(rot_dims // 2)],
+                                                      dtype=torch.float32) if rot_dims else None, persistent=False)
         self.q_norm = _param(dim) if qk_norm else None
         self.k_norm = _param(dim) if qk_norm else None
         self.k_cache = self.v_cache = None            # [pages * block_size, G, d] / [..., G, dv] (values page-transposed), from the runner
@@ -59,14 +74,75 @@ class WindowAttention(nn.Module):
         """Per-token shapes of this layer's K and V pages."""
         return (self.G, self.d), (self.G, self.dv)
 
-    def forward(self, q, k, v, gate) -> torch.Tensor:
+    def forward(self, q, k, v, gate, positions: torch.Tensor | None = None) -> torch.Tensor:
         ctx = get_context()
         ops_seq.knorm_kvstore(k, v, self.k_norm, self.eps, self.G, self.d, self.dv, self.block_size, ctx.slot_mapping, self.k_cache,
-                              self.v_cache)
+                              self.v_cache, positions, self.rot_freq)
         out = torch.empty(q.shape[0], self.H * self.dv, dtype=q.dtype, device=q.device)
         ops_seq.window_attn(q, self.q_norm, self.eps, gate, self.k_cache, self.v_cache, ctx.block_tables, self.block_size,
-                            ctx.portions, self.H, self.G, self.d, self.dv, self.scale, self.window, out)
+                            ctx.portions, self.H, self.G, self.d, self.dv, self.scale, self.window, out, self.chunk, self.rot_freq)
         return out
+
+
+class AttentionMixer(nn.Module):
+    """q | k | v in ONE biased projection, attention (WindowAttention: mask, rotation), out projection."""
+
+    def __init__(self, width: int, heads: int, kv_heads: int, dim: int, vdim: int, scale: float, eps: float, block_size: int,
+                 window: int = 0, chunk: int = 0, rot_dims: int = 0, rot_base: float = 10000.0, qk_norm: bool = False):
+        super().__init__()
+        self.attn = WindowAttention(heads, kv_heads, dim, vdim, scale, window, eps, qk_norm=qk_norm, block_size=block_size,
+                                    chunk=chunk, rot_dims=rot_dims, rot_base=rot_base)
+        self.cols = self.attn.widths[:3]
+        total = sum(self.cols)
+        self.in_w, self.in_b = _param(total, width), _param(total)
+        self.o_w = _param(width, heads * vdim)
+
+    def named_loaders(self) -> dict:
+        q, k, v = self.cols
+        return {"q": _copy_into(self.in_w[:q]), "q.b": _copy_into(self.in_b[:q]), "k": _copy_into(self.in_w[q:q + k]),
+                "k.b": _copy_into(self.in_b[q:q + k]), "v": _copy_into(self.in_w[q + k:]), "v.b": _copy_into(self.in_b[q + k:]),
+                "o": _copy_into(self.o_w)}
+
+    def forward(self, xh: torch.Tensor, positions: torch.Tensor) -> torch.Tensor:
+        proj = F.linear(xh, self.in_w, self.in_b)
+        q, k, v = self.cols
+        return F.linear(self.attn(proj[:, :q], proj[:, q:q + k], proj[:, q + k:], None, positions), self.o_w)
+
+
+class LightningMixer(nn.Module):
+    """Linear attention in its recurrent form: q, k, v = SiLU of the projections; per head S <- decay_h S + k v^T, o = S^T q
+    (state and products in 32-bit); the heads together are RMS-normed (weight `norm`), multiplied by sigmoid(W_g h) and
+    projected. ONE in-projection [v | k | q | g]; SiLU is applied inside the scan as it stages its operands."""
+
+    def __init__(self, width: int, heads: int, dim: int, vdim: int, decay, eps: float):
+        super().__init__()
+        assert len(decay) == heads
+        self.H, self.d, self.dv, self.eps = heads, dim, vdim, eps
+        self.cols = (heads * vdim, heads * dim, heads * dim, heads * vdim)          # v | k | q | g
+        self.in_w = _param(sum(self.cols), width)
+        self.register_buffer("decay", torch.tensor([float(a) for a in decay], dtype=torch.float32), persistent=False)
+        self.norm = _param(heads * vdim)
+        self.o_w = _param(width, heads * vdim)
+        self.rec_state = None
+
+    def state_shapes(self) -> dict:
+        return {"rec_state": (self.H, self.dv, self.d)}
+
+    def named_loaders(self) -> dict:
+        v, k, q, g = self.cols
+        return {"v": _copy_into(self.in_w[:v]), "k": _copy_into(self.in_w[v:v + k]), "q": _copy_into(self.in_w[v + k:v + k + q]),
+                "g": _copy_into(self.in_w[v + k + q:]), "norm": _copy_into(self.norm), "o": _copy_into(self.o_w)}
+
+    def forward(self, xh: torch.Tensor, positions: torch.Tensor | None = None) -> torch.Tensor:
+        por = get_context().portions
+        n = xh.shape[0]
+        v, k, q, g = self.cols
+        proj = F.linear(xh, self.in_w)
+        y = torch.empty(n, v, dtype=torch.float32, device=xh.device)
+        ops_seq.decay_scan(proj, 0, v, v + k, self.decay, self.H, self.d, self.dv, por, self.rec_state, y)
+        out = torch.empty(n, v, dtype=xh.dtype, device=xh.device)
+        ops_seq.gated_group_norm(y, proj[:, v + k + q:], self.norm, 1, self.eps, out, norm_first=True)
+        return F.linear(out, self.o_w)
 
 
 class SSDMixer(nn.Module):
@@ -212,3 +288,86 @@ class XIELUFeedForward(nn.Module):
 
     def forward(self, xh: torch.Tensor) -> torch.Tensor:
         return F.linear(ops_seq.xielu(F.linear(xh, self.up), self.act, self.beta), self.down)
+
+
+class ClampedGLU(nn.Module):
+    """g = min(W_gate h, limit), u = clamp(W_up h, -limit, limit); W_down (g sigmoid(alpha g) (u + 1))."""
+
+    def __init__(self, width: int, ff: int, limit: float, alpha: float = 1.702):
+        super().__init__()
+        self.ff, self.limit, self.alpha = ff, float(limit), float(alpha)
+        self.gu, self.down = _param(2 * ff, width), _param(width, ff)
+
+    def named_loaders(self) -> dict:
+        return {"gate": _copy_into(self.gu[:self.ff]), "up": _copy_into(self.gu[self.ff:]), "down": _copy_into(self.down)}
+
+    def forward(self, xh: torch.Tensor) -> torch.Tensor:
+        gu = F.linear(xh, self.gu)
+        act = torch.empty(xh.shape[0], self.ff, dtype=xh.dtype, device=xh.device)
+        ops_seq.glu_act(gu, self.ff, act, kind=1, limit=self.limit, alpha=self.alpha)
+        return F.linear(act, self.down)
+
+
+class RoutedExperts(nn.Module):
+    """Mixture of `experts` gated feed-forwards W_down (silu(W_gate h) * W_up h), `top` per token.
+
+    Router (32-bit): s = softmax(W_r h) over experts + `identity` pass-through entries (the last ones; their output is h);
+    choice scores s + correction; entries form `group_count` equal groups of neighbours of which the `group_keep` best (by
+    their largest choice score) may be chosen from; weights s[chosen] / sum * `scale`. A shared expert of the same form
+    (`shared_ff`) runs for every token, times sigmoid(w_sg . h). The router's matrix carries w_sg as its last row."""
+
+    def __init__(self, width: int, experts: int, ff: int, top: int, scale: float = 1.0, identity: int = 0, group_count: int = 1,
+                 group_keep: int = 1, shared_ff: int = 0):
+        super().__init__()
+        self.E, self.ident, self.ff, self.top, self.scale = experts, identity, ff, top, float(scale)
+        self.count, self.keep, self.shared_ff = group_count, group_keep, shared_ff
+        total = experts + identity
+        assert total % group_count == 0 and 1 <= group_keep <= group_count and top <= group_keep * (total // group_count)
+        self.router = _param(total + (1 if shared_ff else 0), width, dtype=torch.float32)
+        self.correction = _param(total, dtype=torch.float32)
+        self.w_gu, self.w_down = _param(experts, 2 * ff, width), _param(experts, width, ff)
+        if shared_ff:
+            self.s_gu, self.s_down = _param(2 * shared_ff, width), _param(width, shared_ff)
+
+    def named_loaders(self) -> dict:
+        total, ff = self.E + self.ident, self.ff
+        out = {"router": _copy_into(self.router[:total]), "correction": _copy_into(self.correction)}
+        for e in range(self.E):
+            out[f"e{e}.gate"] = _copy_into(self.w_gu[e, :ff])
+            out[f"e{e}.up"] = _copy_into(self.w_gu[e, ff:])
+            out[f"e{e}.down"] = _copy_into(self.w_down[e])
+        if self.shared_ff:
+            sf = self.shared_ff
+            out.update({"shared.gate": _copy_into(self.s_gu[:sf]), "shared.up": _copy_into(self.s_gu[sf:]),
+                        "shared.down": _copy_into(self.s_down), "shared.sg": _copy_into(self.router[total:])})
+        return out
+
+    def forward(self, xh: torch.Tensor) -> torch.Tensor:
+        n, width = xh.shape
+        total = self.E + self.ident
+        z = F.linear(xh.float(), self.router)                                     # 32-bit, [n, total (+ 1: the shared gate)]
+        ids, wts = ops_seq.moe_route(z, total, self.correction, self.top, self.count, self.keep, self.scale)
+        plan = ops_seq.moe_plan(ids, self.E, 64 if n * self.top >= 64 * self.E else 16)
+        act = torch.empty(plan.cap, self.ff, dtype=xh.dtype, device=xh.device)
+        ops_seq.moe_gemm(xh, self.w_gu, plan, True, act)
+        rows = torch.empty(plan.cap, width, dtype=xh.dtype, device=xh.device)
+        ops_seq.moe_gemm(act, self.w_down, plan, False, rows)
+        shared = gate = None
+        if self.shared_ff:
+            sact = torch.empty(n, self.shared_ff, dtype=xh.dtype, device=xh.device)
+            ops_seq.glu_act(F.linear(xh, self.s_gu), self.shared_ff, sact, kind=0)
+            shared, gate = F.linear(sact, self.s_down), z[:, total:]
+        out = torch.empty(n, width, dtype=xh.dtype, device=xh.device)
+        ops_seq.moe_combine(rows, plan, wts, xh, shared, gate, out)
+        return out
+
+
+def tie_parameters(dst: nn.Module, src: nn.Module) -> None:
+    """Make every parameter of `dst` the SAME tensor as in `src` (two modules of one construction): a layer that runs
+    several times per step with the same weights but caches and state of its own per run."""
+    for name, _ in list(dst.named_parameters()):
+        d, s_ = dst, src
+        parts = name.split(".")
+        for part in parts[:-1]:
+            d, s_ = getattr(d, part), getattr(s_, part)
+        setattr(d, parts[-1], getattr(s_, parts[-1]))

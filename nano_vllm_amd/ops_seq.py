@@ -15,7 +15,7 @@ import torch
 
 from . import build as _build
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 _P, _I, _L, _F = c_void_p, c_int, c_int64, c_float
 
 SIGNATURES = {
@@ -30,11 +30,20 @@ SIGNATURES = {
     "nvs_rglru_scan": (c_int, [_P, _P, _P, _L, _I, _P, _F, _I, _I, _P, _P, _P, _I, _L, _L, _P, _P, _P, _L, _P]),
     "nvs_ssd_scan_workspace": (c_int64, [_I, _I, _I, _I, _L]),
     "nvs_ssd_scan": (c_int, [_P, _P, _L, _L, _I, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _I, _L, _L, _P, _P, _P, _L, _P]),
-    "nvs_gated_group_norm": (c_int, [_P, _P, _L, _I, _P, _I, _I, _F, _L, _P, _P]),
-    "nvs_knorm_kvstore": (c_int, [_P, _P, _L, _I, _P, _F, _I, _I, _I, _I, _P, _L, _P, _P, _P]),
+    "nvs_decay_scan": (c_int, [_P, _L, _L, _L, _L, _I, _P, _I, _I, _I, _P, _P, _P, _I, _L, _L, _P, _P, _P, _L, _P]),
+    "nvs_gated_group_norm": (c_int, [_P, _P, _L, _I, _P, _I, _I, _F, _I, _L, _P, _P]),
+    "nvs_knorm_kvstore": (c_int, [_P, _P, _L, _I, _P, _F, _I, _I, _I, _I, _P, _P, _P, _I, _L, _P, _P, _P]),
     "nvs_window_attn_force_scalar": (None, [_I]),
     "nvs_window_attn": (c_int, [_P, _L, _P, _F, _P, _L, _I, _P, _P, _P, _L, _I, _P, _P, _P, _I, _L, _I, _I, _I, _I, _F, _I,
-                                _P, _P]),
+                                _I, _P, _I, _P, _P]),
+    "nvs_add_group_norm": (c_int, [_P, _P, _P, _P, _L, _P, _I, _I, _I, _F, _P, _P]),
+    "nvs_glu_act": (c_int, [_P, _L, _I, _I, _I, _F, _F, _L, _P, _P]),
+    "nvs_moe_route": (c_int, [_P, _L, _P, _L, _I, _I, _I, _I, _F, _P, _P, _P]),
+    "nvs_moe_rows": (c_int64, [_L, _I, _I]),
+    "nvs_moe_plan": (c_int, [_P, _L, _I, _I, _I, _P, _P, _P, _P]),
+    "nvs_moe_gemm": (c_int, [_P, _L, _P, _I, _I, _I, _I, _P, _P, _L, _I, _P, _L, _P]),
+    "nvs_moe_force_plain": (None, [_I]),
+    "nvs_moe_combine": (c_int, [_P, _L, _P, _P, _I, _P, _L, _P, _P, _L, _I, _L, _I, _P, _P]),
 }
 
 _lib = None
@@ -192,17 +201,27 @@ def ssd_scan(xbc: torch.Tensor, proj: torch.Tensor, dt_col: int, dt_bias, A_log,
                             por.max_q, _ptr(S), _ptr(y), _ptr(ws), need, _stream()))
 
 
-def gated_group_norm(y: torch.Tensor, z: torch.Tensor, w: torch.Tensor, groups: int, eps: float, out: torch.Tensor):
+def gated_group_norm(y: torch.Tensor, z: torch.Tensor, w: torch.Tensor, groups: int, eps: float, out: torch.Tensor,
+                     norm_first: bool = False):
+    """out = group_rms(y * silu(z)) * w, or with norm_first group_rms(y) * w * sigmoid(z)."""
     lib = load_library()
     n, inner = y.shape
     assert y.dtype == torch.float32 and y.is_contiguous() and z.shape == (n, inner) and z.stride(1) == 1
     assert w.numel() == inner and out.shape == (n, inner) and out.is_contiguous()
-    _check(lib.nvs_gated_group_norm(_ptr(y), _ptr(z), z.stride(0), _same(z, w, out), _ptr(w), inner, groups, eps, n, _ptr(out),
-                                    _stream()))
+    _check(lib.nvs_gated_group_norm(_ptr(y), _ptr(z), z.stride(0), _same(z, w, out), _ptr(w), inner, groups, eps, int(norm_first), n,
+                                    _ptr(out), _stream()))
+
+
+def _rotation(rot_freq: torch.Tensor | None) -> int:
+    if rot_freq is None:
+        return 0
+    assert rot_freq.dtype == torch.float32 and rot_freq.is_contiguous() and rot_freq.is_cuda
+    return 2 * rot_freq.numel()
 
 
 def knorm_kvstore(k: torch.Tensor, v: torch.Tensor, knorm: torch.Tensor | None, eps: float, G: int, d: int, dv: int,
-                  block_size: int, slots: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor):
+                  block_size: int, slots: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                  pos: torch.Tensor | None = None, rot_freq: torch.Tensor | None = None):
     """k [n, G*d], v [n, G*dv]: column ranges of ONE projection output (same row stride). v_cache has the shape
     [pages * block_size, G, dv] but is laid out [page][G][dv][block_size] (see include/nvl_seq.h)."""
     assert k_cache.shape[0] % block_size == 0
@@ -212,13 +231,17 @@ def knorm_kvstore(k: torch.Tensor, v: torch.Tensor, knorm: torch.Tensor | None, 
     assert slots.dtype == torch.int32 and slots.numel() >= n
     assert k_cache.is_contiguous() and v_cache.is_contiguous()
     assert tuple(k_cache.shape[1:]) == (G, d) and tuple(v_cache.shape[1:]) == (G, dv)
+    assert rot_freq is None or (pos is not None and pos.dtype == torch.int64 and pos.numel() >= n and pos.is_contiguous())
     _check(lib.nvs_knorm_kvstore(_ptr(k), _ptr(v), k.stride(0), _same(k, v, knorm, k_cache, v_cache), _ptr(knorm), eps, G, d, dv,
-                                 block_size, _ptr(slots), n, _ptr(k_cache), _ptr(v_cache), _stream()))
+                                 block_size, _ptr(slots), _ptr(pos) if rot_freq is not None else None, _ptr(rot_freq),
+                                 _rotation(rot_freq), n, _ptr(k_cache), _ptr(v_cache), _stream()))
 
 
 def window_attn(q: torch.Tensor, qnorm: torch.Tensor | None, eps: float, gate: torch.Tensor | None, k_cache, v_cache,
                 block_tables: torch.Tensor, block_size: int, por: Portions, H: int, G: int, d: int, dv: int, scale: float,
-                window: int, out: torch.Tensor):
+                window: int, out: torch.Tensor, chunk: int = 0, rot_freq: torch.Tensor | None = None):
+    """window > 0: the last `window` positions; chunk > 0: the query's own block of `chunk` positions; neither: causal.
+    rot_freq [r / 2] (32-bit): the first r entries of every query head turn in interleaved pairs by position * rot_freq."""
     lib = load_library()
     n = por.n
     assert q.shape == (n, H * d) and q.stride(1) == 1 and out.shape == (n, H * dv) and out.is_contiguous()
@@ -228,4 +251,107 @@ def window_attn(q: torch.Tensor, qnorm: torch.Tensor | None, eps: float, gate: t
     _check(lib.nvs_window_attn(_ptr(q), q.stride(0), _ptr(qnorm), eps, _ptr(gate), gate.stride(0) if gate is not None else 0,
                                _same(q, qnorm, gate, k_cache, v_cache, out), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
                                block_tables.stride(0), block_size, _ptr(por.cu_q), _ptr(por.ctx0), _ptr(por.tseq), por.nseq, n, H,
-                               G, d, dv, scale, window, _ptr(out), _stream()))
+                               G, d, dv, scale, window, chunk, _ptr(rot_freq), _rotation(rot_freq), _ptr(out), _stream()))
+
+
+def add_group_norm(x: torch.Tensor, w: torch.Tensor | None, groups: int, eps: float, out: torch.Tensor | None,
+                   a: torch.Tensor | None = None, b: torch.Tensor | None = None):
+    """x += a + b (in place; a in the activation type, b 32-bit, both optional), then out = group_rms(x) * w (out None: adds only)."""
+    lib = load_library()
+    n, width = x.shape
+    assert x.dtype == torch.float32 and x.is_contiguous()
+    assert a is None or (a.shape == x.shape and a.is_contiguous())
+    assert b is None or (b.shape == x.shape and b.is_contiguous() and b.dtype == torch.float32)
+    assert out is None or (out.shape == x.shape and out.is_contiguous() and w is not None and w.numel() == width)
+    ref = out if out is not None else a
+    assert ref is not None, "nothing to do"
+    _check(lib.nvs_add_group_norm(_ptr(x), _ptr(a), _ptr(b), None, n, _ptr(w) if out is not None else None, _same(ref, a, w, out), width,
+                                  groups, eps, _ptr(out), _stream()))
+
+
+def group_norm_rows(x: torch.Tensor, rows: torch.Tensor | None, nrows: int, w: torch.Tensor, groups: int, eps: float, out: torch.Tensor):
+    """out[r] = group_rms(x[rows[r]]) * w (rows None: row r)."""
+    lib = load_library()
+    assert x.dtype == torch.float32 and x.is_contiguous() and out.is_contiguous() and out.shape == (nrows, x.shape[1])
+    assert rows is None or (rows.dtype == torch.int32 and rows.numel() >= nrows)
+    assert rows is not None or nrows <= x.shape[0]
+    _check(lib.nvs_add_group_norm(_ptr(x), None, None, _ptr(rows), nrows, _ptr(w), _same(out, w), x.shape[1], groups, eps, _ptr(out),
+                                  _stream()))
+
+
+def decay_scan(proj: torch.Tensor, v_col: int, k_col: int, q_col: int, decay: torch.Tensor, heads: int, dk: int, dv: int,
+               por: Portions, S: torch.Tensor, y: torch.Tensor):
+    """Per head S = decay S + k v^T, y = S^T q on SiLU of the named columns of proj; S [nslots, heads, dv, dk], y [n, heads * dv]."""
+    lib = load_library()
+    n = por.n
+    assert proj.shape[0] == n and proj.stride(1) == 1
+    assert decay.dtype == torch.float32 and decay.numel() == heads and decay.is_contiguous()
+    assert S.dtype == torch.float32 and S.is_contiguous() and tuple(S.shape[1:]) == (heads, dv, dk)
+    assert y.dtype == torch.float32 and y.is_contiguous() and y.shape == (n, heads * dv)
+    need = 0 if torch.cuda.is_current_stream_capturing() else lib.nvs_ssd_scan_workspace(heads, dv, dk, por.nseq, por.max_q)
+    ws = torch.empty(need, dtype=torch.float32, device=proj.device) if need else None
+    _check(lib.nvs_decay_scan(_ptr(proj), proj.stride(0), v_col, k_col, q_col, _code(proj), _ptr(decay), heads, dk, dv, _ptr(por.cu_q),
+                              _ptr(por.ctx0), _ptr(por.slot), por.nseq, n, por.max_q, _ptr(S), _ptr(y), _ptr(ws), need, _stream()))
+
+
+def glu_act(gu: torch.Tensor, ff: int, out: torch.Tensor, kind: int = 0, limit: float = 0.0, alpha: float = 1.0):
+    """gu [n, 2 ff] = [gate | up] -> out [n, ff]. kind 0: silu(g) u; kind 1: min(g, limit) sigmoid(alpha g) (clamp(u) + 1)."""
+    lib = load_library()
+    n = gu.shape[0]
+    assert gu.shape[1] == 2 * ff and gu.stride(1) == 1 and out.shape == (n, ff) and out.is_contiguous()
+    _check(lib.nvs_glu_act(_ptr(gu), gu.stride(0), _same(gu, out), ff, kind, limit, alpha, n, _ptr(out), _stream()))
+
+
+def moe_route(z: torch.Tensor, total: int, correction: torch.Tensor | None, top: int, count: int, keep: int, scale: float):
+    """z [n, >= total] 32-bit router logits -> (ids [n, top] int32, weights [n, top] 32-bit)."""
+    lib = load_library()
+    n = z.shape[0]
+    assert z.dtype == torch.float32 and z.stride(1) == 1 and z.shape[1] >= total
+    assert correction is None or (correction.dtype == torch.float32 and correction.numel() == total and correction.is_contiguous())
+    ids = torch.empty(n, top, dtype=torch.int32, device=z.device)
+    wts = torch.empty(n, top, dtype=torch.float32, device=z.device)
+    _check(lib.nvs_moe_route(_ptr(z), z.stride(0), _ptr(correction), n, total, top, count, keep, scale, _ptr(ids), _ptr(wts), _stream()))
+    return ids, wts
+
+
+class MoePlan:
+    __slots__ = ("tile_expert", "row_token", "pair_row", "cap", "tm")
+
+
+def moe_plan(ids: torch.Tensor, experts: int, tm: int) -> MoePlan:
+    """Pairs (token, choice) sorted by expert into tiles of tm rows (ids >= experts get no row)."""
+    lib = load_library()
+    n, top = ids.shape
+    assert ids.dtype == torch.int32 and ids.is_contiguous()
+    p = MoePlan()
+    p.tm, p.cap = tm, lib.nvs_moe_rows(n * top, experts, tm)
+    p.tile_expert = torch.empty(p.cap // tm, dtype=torch.int32, device=ids.device)
+    p.row_token = torch.empty(p.cap, dtype=torch.int32, device=ids.device)
+    p.pair_row = torch.empty(n, top, dtype=torch.int32, device=ids.device)
+    _check(lib.nvs_moe_plan(_ptr(ids), n, top, experts, tm, _ptr(p.tile_expert), _ptr(p.row_token), _ptr(p.pair_row), _stream()))
+    return p
+
+
+def moe_gemm(x: torch.Tensor, w: torch.Tensor, plan: MoePlan, glu: bool, out: torch.Tensor):
+    """glu: w [experts, 2 nout, K], rows gathered by token, out = silu(gate) * up; else w [experts, nout, K], x holds the planned rows."""
+    lib = load_library()
+    nout, K = (w.shape[1] // 2 if glu else w.shape[1]), w.shape[2]
+    assert w.is_contiguous() and x.stride(1) == 1 and x.shape[1] == K and out.shape == (plan.cap, nout) and out.stride(1) == 1
+    assert glu or x.shape[0] == plan.cap
+    _check(lib.nvs_moe_gemm(_ptr(x), x.stride(0), _ptr(w), _same(x, w, out), int(glu), nout, K, _ptr(plan.tile_expert), _ptr(plan.row_token),
+                            plan.cap, plan.tm, _ptr(out), out.stride(0), _stream()))
+
+
+def moe_combine(rows: torch.Tensor, plan: MoePlan, wts: torch.Tensor, h: torch.Tensor, shared: torch.Tensor | None,
+                shared_gate: torch.Tensor | None, out: torch.Tensor):
+    """out[t] = sum_k wts[t, k] * (row of the pair, or h[t] for a pass-through choice) + sigmoid(shared_gate[t]) * shared[t]."""
+    lib = load_library()
+    n, width = h.shape
+    top = wts.shape[1]
+    assert rows.stride(1) == 1 and rows.shape[1] == width and h.stride(1) == 1 and out.shape == (n, width) and out.is_contiguous()
+    assert wts.dtype == torch.float32 and wts.is_contiguous() and plan.pair_row.shape == (n, top)
+    assert shared is None or (shared.shape == (n, width) and shared.is_contiguous() and shared_gate.dtype == torch.float32
+                              and shared_gate.shape[0] == n)
+    _check(lib.nvs_moe_combine(_ptr(rows), rows.stride(0), _ptr(plan.pair_row), _ptr(wts), top, _ptr(h), h.stride(0), _ptr(shared),
+                               _ptr(shared_gate), shared_gate.stride(0) if shared_gate is not None else 0, _same(rows, h, shared, out), n,
+                               width, _ptr(out), _stream()))

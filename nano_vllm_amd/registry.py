@@ -48,10 +48,22 @@ def _foduzen_build(config, dtype=None):
     return FoduzenForCausalLM(config, dtype)
 
 
+def _nokipel_config(path: str, raw: dict):
+    from .nokipel import NokipelConfig
+    return NokipelConfig(raw)
+
+
+def _nokipel_build(config, dtype=None):
+    from .nokipel import NokipelForCausalLM
+    return NokipelForCausalLM(config, dtype)
+
+
 REGISTRY: dict[str, ModelSpec] = {
     "Qwen3ForCausalLM": ModelSpec("Qwen3ForCausalLM", _qwen3_config, _qwen3_build),
     "Qwen2ForCausalLM": ModelSpec("Qwen2ForCausalLM", _qwen3_config, _qwen3_build),      # same module tree, biased qkv, no q/k norm
     "Foduzen": ModelSpec("Foduzen", _foduzen_config, _foduzen_build, stateful=True, block_multiple=16,
+                         dtypes=("bfloat16", "float32")),
+    "Nokipel": ModelSpec("Nokipel", _nokipel_config, _nokipel_build, stateful=True, block_multiple=16,
                          dtypes=("bfloat16", "float32")),
 }
 
