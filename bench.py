@@ -29,9 +29,9 @@ driver's fields it carries
                  race keys with the draws replayed (a by-product of the cpu_baseline leg: the timed
                  oracle pass is teacher-forced with the engine's tokens).
 
-`python bench.py --compare-families [--families foduzen,qwen3] [--sizes 1k,4k]` is a different measurement with a line of
-its own (metric "family_compare"): prefill and decode throughput of the Foduzen family at layer sizes of real models beside
-Qwen3 at equal width and depth. The default command above is unchanged by it.
+`python bench.py --compare-families [--families nokipel,foduzen,qwen3] [--sizes 1k,4k]` is a different measurement with a line
+of its own (metric "family_compare"): prefill and decode throughput of the Nokipel and Foduzen families at layer sizes of real
+models beside Qwen3 at equal width and depth. The default command above is unchanged by it.
 """
 from __future__ import annotations
 
@@ -89,9 +89,9 @@ def parse():
     ap.add_argument("--kv-cache-dtype", default="bf16", choices=["bf16", "fp8"],
                     help="fp8: opt-in OCP e4m3 KV cache (outside the reference's numerics; never the headline)")
     ap.add_argument("--compare-families", action="store_true",
-                    help="instead of the headline workload: prefill and decode throughput of the Foduzen family at layer sizes of "
-                         "real models (random weights) beside Qwen3 models of equal width / depth, one JSON line")
-    ap.add_argument("--families", default="foduzen,qwen3", help="with --compare-families: which of the two to run")
+                    help="instead of the headline workload: prefill and decode throughput of the Nokipel and Foduzen families at "
+                         "layer sizes of real models (random weights) beside Qwen3 models of equal width / depth, one JSON line")
+    ap.add_argument("--families", default="nokipel,foduzen,qwen3", help="with --compare-families: which of the three to run")
     ap.add_argument("--sizes", default="1k,4k", help="with --compare-families: layer sizes to run (1k, 4k)")
     return ap.parse_args()
 
@@ -106,6 +106,24 @@ def foduzen_config(width: int, ff: int, heads: int, kv_heads: int, layers: int, 
     rec = {"type": "rglru", "mlp": {"kind": "dense", "ff": ff}, "mixer": {"width": width, "blocks": width // 128, "conv": 4}}
     return {"architecture": "Foduzen", "embedding": {"scale": 1.0}, "layers": [par if i % 2 == 0 else rec for i in range(layers)],
             "norm": {"eps": 1e-6}, "vocab": vocab, "width": width}
+
+
+def nokipel_config(width: int, ff: int, heads: int, kv_heads: int, layers: int, vocab: int) -> dict:
+    """Layers of a real model's size: 128-wide attention heads in blocks of 1,024 positions with half of every head rotated,
+    128 x 128 lightning heads (as many as make the model's width), a routed feed-forward whose three chosen experts and shared
+    expert together are as wide as the dense one (30 experts + 2 pass-through entries in 4 groups, 2 kept); attention + routed
+    and lightning + dense layers alternate."""
+    eff = ff // 4
+    att = {"type": "attention",
+           "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "mask": {"size": 1024},
+                     "rot": {"dims": 64, "base": 500000.0}},
+           "mlp": {"kind": "moe", "expert": {"ff": eff}, "shared": {"ff": eff},
+                   "router": {"experts": 30, "identity": 2, "top": 3, "scale": 1.0, "groups": {"count": 4, "keep": 2}}}}
+    nh = width // 128
+    lig = {"type": "lightning", "mlp": {"kind": "dense", "ff": ff, "limit": 7.0},
+           "mixer": {"heads": nh, "dim": 128, "vdim": 128, "decay": [1.0 - 2.0 ** (-3 - 5 * i / max(nh - 1, 1)) for i in range(nh)]}}
+    return {"architecture": "Nokipel", "embedding": {"scale": 1.0}, "layers": [att if i % 2 == 0 else lig for i in range(layers)],
+            "norm": {"eps": 1e-6, "groups": 1}, "vocab": vocab, "width": width}
 
 
 FAMILY_SIZES = {   # name: (width, ff, heads, kv heads, layers, the Qwen3 shape of the same width / depth)
@@ -129,8 +147,8 @@ def compare_families(args) -> dict:
         width, ff, heads, kv, layers, qname = FAMILY_SIZES[size]
         for family in args.families.split(","):
             path = os.path.join(tempfile.gettempdir(), f"nvl_cmp_{family}_{size}")
-            if family == "foduzen":
-                raw = foduzen_config(width, ff, heads, kv, layers, vocab)
+            if family in ("foduzen", "nokipel"):
+                raw = (foduzen_config if family == "foduzen" else nokipel_config)(width, ff, heads, kv, layers, vocab)
                 os.makedirs(path, exist_ok=True)
                 with open(os.path.join(path, "config.json"), "w") as fh:
                     json.dump(raw, fh)

@@ -173,3 +173,76 @@ def test_checkpoint_names_and_the_models_loaders_agree():
     assert model.layers[0].mlp is None and model.layers[0].norm2 is None
     with pytest.raises(AssertionError):
         loaders["embed"](torch.zeros(3, 3))
+
+
+# ---- Nokipel: configuration, layer runs, shared weights, checkpoint names (no GPU) -----------------------------------
+def nkp_raw():
+    light = {"type": "lightning", "mixer": {"heads": 2, "dim": 8, "vdim": 12, "decay": [0.5, 0.99]}, "mlp": {"kind": "dense", "ff": 20, "limit": 2.0}}
+    attn = {"type": "attention", "mixer": {"heads": 4, "kv_heads": 2, "dim": 8, "vdim": 6, "scale": 0.3, "mask": {"size": 5},
+                                           "rot": {"dims": 4, "base": 100.0}},
+            "mlp": {"kind": "moe", "expert": {"ff": 10}, "shared": {"ff": 14},
+                    "router": {"experts": 3, "identity": 1, "top": 2, "scale": 1.5, "groups": {"count": 2, "keep": 1}}}}
+    bare = {"type": "attention", "mixer": {"heads": 2, "kv_heads": 2, "dim": 6, "vdim": 6, "scale": 0.4}, "mlp": None}
+    return {"architecture": "Nokipel", "embedding": {"scale": 2.0}, "layers": [light, attn, bare, light], "loop": {"start": 1, "stop": 3, "times": 3},
+            "norm": {"eps": 1e-5, "groups": 2}, "vocab": 29, "width": 16}
+
+
+def test_nokipel_registry_config_and_order_of_layer_runs(tmp_path):
+    from nano_vllm_amd.registry import REGISTRY, resolve
+    (tmp_path / "config.json").write_text(json.dumps(nkp_raw()))
+    spec, cfg = resolve(str(tmp_path))
+    assert spec is REGISTRY["Nokipel"] and spec.stateful and set(spec.dtypes) == {"bfloat16", "float32"}
+    assert cfg.vocab_size == 29 and cfg.hidden_size == 16 and cfg.norm_groups == 2
+    assert cfg.runs() == [(0, 0), (1, 0), (2, 0), (1, 1), (2, 1), (1, 2), (2, 2), (3, 0)]
+    raw = nkp_raw()
+    del raw["loop"]
+    (tmp_path / "config.json").write_text(json.dumps(raw))
+    assert resolve(str(tmp_path))[1].runs() == [(0, 0), (1, 0), (2, 0), (3, 0)]
+    for key, bad, msg in (("type", "lstm", "mixer type"), ("mlp", {"kind": "conv"}, "feed-forward kind")):
+        raw = nkp_raw()
+        raw["layers"][0][key] = bad
+        (tmp_path / "config.json").write_text(json.dumps(raw))
+        with pytest.raises(ValueError, match=msg):
+            resolve(str(tmp_path))
+    raw = nkp_raw()
+    raw["loop"]["stop"] = 9
+    (tmp_path / "config.json").write_text(json.dumps(raw))
+    with pytest.raises(ValueError, match="loop"):
+        resolve(str(tmp_path))
+
+
+def test_nokipel_checkpoint_names_loaders_and_weights_shared_between_runs():
+    """Every tensor the synthetic checkpoint writes has a loader in the model and the other way round; a layer inside the
+    repeated span has one mixer per run, all on the SAME weight tensors, each with cache / state attributes of its own."""
+    from nano_vllm_amd.nokipel import NokipelConfig, NokipelForCausalLM, random_tensors, tensor_shapes
+    raw = nkp_raw()
+    model = NokipelForCausalLM(NokipelConfig(raw), torch.float32, block_size=16)
+    loaders = model.named_loaders()
+    shapes = tensor_shapes(raw)
+    assert set(loaders) == set(shapes)
+    tensors = random_tensors(raw, seed=3)
+    with torch.no_grad():
+        for name, t in tensors.items():
+            assert tuple(t.shape) == tuple(shapes[name]) and t.dtype == torch.bfloat16
+            loaders[name](t)
+    assert [len(layer.mixers) for layer in model.layers] == [1, 3, 3, 1]
+    a = model.layers[1].mixers
+    assert a[0].in_w is a[1].in_w is a[2].in_w and a[0].o_w is a[2].o_w and a[0].attn is not a[2].attn
+    q, k, v = a[0].cols
+    assert (q, k, v) == (32, 16, 12) and torch.equal(a[2].in_w[q:q + k], tensors["l1.mix.k"].float())
+    assert torch.equal(a[1].in_b[q + k:], tensors["l1.mix.v.b"].float())
+    assert a[0].attn.chunk == 5 and a[0].attn.window == 0 and a[0].attn.rot_freq.tolist() == [1.0, pytest.approx(0.1)]
+    assert model.layers[2].mixers[0].attn.chunk == 0 and model.layers[2].mixers[0].attn.rot_freq is None and model.layers[2].mlp is None
+    kv_layers = [m for m in model.modules() if hasattr(m, "kv_shapes")]
+    st_layers = [m for m in model.modules() if hasattr(m, "state_shapes")]
+    assert len(kv_layers) == 6 and len(st_layers) == 2 and st_layers[0].state_shapes() == {"rec_state": (2, 12, 8)}
+    n_params = sum(p.numel() for p in model.parameters())                     # shared tensors count once
+    assert n_params == sum(int(torch.tensor(s).prod()) for s in shapes.values())
+    lig = model.layers[0].mixers[0]
+    v, k, q, g = lig.cols
+    assert torch.equal(lig.in_w[v + k:v + k + q], tensors["l0.mix.q"].float()) and lig.decay.tolist() == [0.5, pytest.approx(0.99)]
+    moe = model.layers[1].mlp
+    assert moe.router.dtype == torch.float32 and moe.router.shape == (5, 16) and torch.equal(moe.router[4:], tensors["l1.mlp.shared.sg"].float())
+    assert torch.equal(moe.w_gu[2, 10:], tensors["l1.mlp.e2.up"].float()) and moe.correction.dtype == torch.float32
+    with pytest.raises(AssertionError):
+        loaders["embed"](torch.zeros(3, 3))
