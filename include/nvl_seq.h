@@ -138,7 +138,7 @@ int nvs_moe_route(const float* z, int64_t z_stride, const float* correction, int
                   int32_t* ids, float* wts, void* stream);
 
 /* Sort the pairs (token, choice) by expert. Pairs whose id >= experts have no rows (pass-through entries). Every expert's rows are
- * padded to whole tiles of tm (16 or 64) rows; cap = nvs_moe_rows(n * top, experts, tm) rows are laid out.
+ * padded to whole tiles of tm (16, 64 or 128) rows; cap = nvs_moe_rows(n * top, experts, tm) rows are laid out.
  * tile_expert [cap / tm]: the tile's expert or -1; row_token [cap]: the row's token or -1; pair_row [n * top]: the pair's row or -1. */
 int64_t nvs_moe_rows(int64_t pairs, int experts, int tm);
 int nvs_moe_plan(const int32_t* ids, int64_t n, int top, int experts, int tm, int32_t* tile_expert, int32_t* row_token, int32_t* pair_row,
@@ -146,7 +146,8 @@ int nvs_moe_plan(const int32_t* ids, int64_t n, int top, int experts, int tm, in
 
 /* Grouped product over the planned rows: out[r, :] = W[expert of r] x(r). glu != 0: W [experts, 2 nout, K] (gate rows, then up rows),
  * x(r) = X[row_token[r], :], out = silu(gate) * up; glu == 0: W [experts, nout, K], x(r) = X[r, :]. X, W, out in `dtype`; bf16 with
- * K % 8 == 0 and ldx % 8 == 0 runs on the matrix cores. Padding rows are not written. */
+ * K % 8 == 0 and ldx % 8 == 0 runs on the matrix cores (tm 128: LDS-tiled, for steps with many rows per expert). Padding rows are
+ * not written. */
 int nvs_moe_gemm(const void* X, int64_t ldx, const void* W, int dtype, int glu, int nout, int K, const int32_t* tile_expert,
                  const int32_t* row_token, int64_t cap, int tm, void* out, int64_t ldo, void* stream);
 /* tests: 1 routes bf16 calls through the plain kernel as well */

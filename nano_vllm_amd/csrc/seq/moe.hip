@@ -289,6 +289,103 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(const bf16_t* __rest
   }
 }
 
+// LDS-tiled matrix-core form for steps with many rows per expert (tiles of 128 rows). A workgroup of four wavefronts computes
+// 128 rows x 128 features (GLU: gate and up of the same 128 features, 256 weight rows) in steps of 32 along k: all threads
+// load the step's operands with 16-byte loads — the NEXT step's loads are issued before the current step is computed — into
+// LDS as [row][32 + 8]; a wavefront owns 64 rows x 64 features (4 x 4 MFMA tiles per operand set) and reads its operands as
+// 16-byte LDS reads: 8 (12) reads for 16 (32) MFMAs. The grid is one-dimensional and XCD-aware: workgroups are dealt to the
+// eight XCDs round-robin, so workgroup id -> (id % 8) * per_xcd + id / 8 gives every XCD a CONTIGUOUS run of tiles, ordered
+// feature tile major / row tile minor: consecutive tiles of an XCD share a weight tile (all row tiles of one expert), which
+// its L2 then serves.
+template <bool GLU>
+__global__ __launch_bounds__(256) void moe_gemm_tiled_kernel(const bf16_t* __restrict__ X, int64_t ldx, const bf16_t* __restrict__ W, int nout,
+                                                             int K, const int32_t* __restrict__ tile_expert,
+                                                             const int32_t* __restrict__ row_token, int tiles_m, int tiles_n,
+                                                             bf16_t* __restrict__ out, int64_t ldo) {
+  constexpr int BM = 128, BN = 128, BK = 32, LDK = BK + 8, NG = GLU ? 2 : 1;
+  __shared__ __attribute__((aligned(16))) bf16_t Xs[BM][LDK];
+  __shared__ __attribute__((aligned(16))) bf16_t Ws[NG * BN][LDK];
+  const int per_xcd = gridDim.x / 8;
+  const int logical = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+  if (logical >= tiles_m * tiles_n) return;
+  const int rt = logical % tiles_m, ft = logical / tiles_m;
+  const int e = tile_expert[rt];
+  if (e < 0) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, lk = (lane >> 4) * 8;
+  const int wm = wave & 1, wn = wave >> 1;
+  const int64_t row0 = (int64_t)rt * BM;
+  const bf16_t* We = W + (int64_t)e * NG * nout * K;
+  // staging: unit u = tid + 256 i -> (row u >> 2, 8 elements of k at (u & 3) * 8)
+  const int sk = (tid & 3) * 8;
+  const bf16_t* xsrc[2];
+  const bf16_t* wsrc[2 * NG];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int r = (tid >> 2) + 64 * i;
+    const int tok = row_token[row0 + r];
+    xsrc[i] = tok >= 0 ? X + (GLU ? (int64_t)tok : row0 + r) * ldx + sk : nullptr;
+  }
+#pragma unroll
+  for (int i = 0; i < 2 * NG; ++i) {
+    const int r = (tid >> 2) + 64 * i, g = r / BN, f = ft * BN + r % BN;
+    wsrc[i] = f < nout ? We + ((int64_t)g * nout + f) * K + sk : nullptr;
+  }
+  const u32x4_t zero4 = u32x4_t{0u, 0u, 0u, 0u};
+  u32x4_t xr[2], wr[2 * NG];
+  auto fetch = [&](int k0) {
+    const bool kin = k0 + sk < K;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) xr[i] = (kin && xsrc[i]) ? *(const u32x4_t*)(xsrc[i] + k0) : zero4;
+#pragma unroll
+    for (int i = 0; i < 2 * NG; ++i) wr[i] = (kin && wsrc[i]) ? *(const u32x4_t*)(wsrc[i] + k0) : zero4;
+  };
+  f32x4_t acc[NG][4][4];
+#pragma unroll
+  for (int g = 0; g < NG; ++g)
+#pragma unroll
+    for (int fb = 0; fb < 4; ++fb)
+#pragma unroll
+      for (int rb = 0; rb < 4; ++rb) acc[g][fb][rb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  fetch(0);
+  for (int k0 = 0; k0 < K; k0 += BK) {
+    __syncthreads();                                // the previous step's readers are done
+#pragma unroll
+    for (int i = 0; i < 2; ++i) *(u32x4_t*)&Xs[(tid >> 2) + 64 * i][sk] = xr[i];
+#pragma unroll
+    for (int i = 0; i < 2 * NG; ++i) *(u32x4_t*)&Ws[(tid >> 2) + 64 * i][sk] = wr[i];
+    __syncthreads();
+    if (k0 + BK < K) fetch(k0 + BK);
+    bf16x8_t xb[4];
+#pragma unroll
+    for (int rb = 0; rb < 4; ++rb) xb[rb] = *(const bf16x8_t*)&Xs[wm * 64 + rb * 16 + li][lk];
+#pragma unroll
+    for (int g = 0; g < NG; ++g)
+#pragma unroll
+      for (int fb = 0; fb < 4; ++fb) {
+        const bf16x8_t wa = *(const bf16x8_t*)&Ws[g * BN + wn * 64 + fb * 16 + li][lk];
+#pragma unroll
+        for (int rb = 0; rb < 4; ++rb) acc[g][fb][rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa, xb[rb], acc[g][fb][rb], 0, 0, 0);
+      }
+  }
+  // lane: row li of row block rb, features 16 fb + 4 (lane >> 4) + 0..3 of its wavefront's 64
+#pragma unroll
+  for (int rb = 0; rb < 4; ++rb) {
+    const int64_t r = row0 + wm * 64 + rb * 16 + li;
+    if (row_token[r] < 0) continue;
+#pragma unroll
+    for (int fb = 0; fb < 4; ++fb) {
+      const int f = ft * BN + wn * 64 + fb * 16 + (lane >> 4) * 4;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (f + i < nout) {
+          const float v = GLU ? glu_value(acc[0][fb][rb][i], acc[NG - 1][fb][rb][i], 0, 0.f, 0.f) : acc[0][fb][rb][i];
+          out[r * ldo + f + i] = (bf16_t)v;
+        }
+      }
+    }
+  }
+}
+
 // ---- combine: one workgroup per token ------------------------------------------------------------------------------------
 template <typename T>
 __global__ void moe_combine_kernel(const T* __restrict__ rows, int64_t ldr, const int32_t* __restrict__ pair_row,
@@ -343,7 +440,7 @@ extern "C" int64_t nvs_moe_rows(int64_t pairs, int experts, int tm) { return (pa
 extern "C" int nvs_moe_plan(const int32_t* ids, int64_t n, int top, int experts, int tm, int32_t* tile_expert, int32_t* row_token,
                             int32_t* pair_row, void* stream) {
   NVS_REQUIRE(ids && tile_expert && row_token && pair_row && n >= 0 && top > 0, "nvs_moe_plan: null argument");
-  NVS_REQUIRE(experts > 0 && experts <= MAX_EXPERTS && (tm == 16 || tm == 64), "nvs_moe_plan: %d experts, tiles of %d rows", experts, tm);
+  NVS_REQUIRE(experts > 0 && experts <= MAX_EXPERTS && (tm == 16 || tm == 64 || tm == 128), "nvs_moe_plan: %d experts, tiles of %d rows", experts, tm);
   if (n == 0) return NVS_OK;
   const int64_t cap = nvs_moe_rows(n * top, experts, tm);
   NVS_REQUIRE(cap < (1ll << 31), "nvs_moe_plan: step too large");
@@ -354,10 +451,22 @@ extern "C" int nvs_moe_plan(const int32_t* ids, int64_t n, int top, int experts,
 extern "C" int nvs_moe_gemm(const void* X, int64_t ldx, const void* W, int dtype, int glu, int nout, int K, const int32_t* tile_expert,
                             const int32_t* row_token, int64_t cap, int tm, void* out, int64_t ldo, void* stream) {
   NVS_REQUIRE(X && W && tile_expert && row_token && out, "nvs_moe_gemm: null argument");
-  NVS_REQUIRE(nout > 0 && K > 0 && ldx >= K && ldo >= nout && (tm == 16 || tm == 64) && cap >= 0 && cap % tm == 0,
+  NVS_REQUIRE(nout > 0 && K > 0 && ldx >= K && ldo >= nout && (tm == 16 || tm == 64 || tm == 128) && cap >= 0 && cap % tm == 0,
               "nvs_moe_gemm: %d x %d, %lld rows in tiles of %d", nout, K, (long long)cap, tm);
   if (cap == 0) return NVS_OK;
   hipStream_t st = (hipStream_t)stream;
+  if (dtype == NVS_BF16 && K % 8 == 0 && ldx % 8 == 0 && !g_moe_plain && tm == 128) {
+    const int tiles_m = (int)(cap / 128), tiles_n = (nout + 127) / 128;
+    const int64_t blocks = ((int64_t)tiles_m * tiles_n + 7) / 8 * 8;
+    NVS_REQUIRE(blocks < (1ll << 31), "nvs_moe_gemm: step too large");
+    if (glu)
+      moe_gemm_tiled_kernel<true><<<dim3((unsigned)blocks), dim3(256), 0, st>>>((const bf16_t*)X, ldx, (const bf16_t*)W, nout, K, tile_expert,
+                                                                                row_token, tiles_m, tiles_n, (bf16_t*)out, ldo);
+    else
+      moe_gemm_tiled_kernel<false><<<dim3((unsigned)blocks), dim3(256), 0, st>>>((const bf16_t*)X, ldx, (const bf16_t*)W, nout, K, tile_expert,
+                                                                                 row_token, tiles_m, tiles_n, (bf16_t*)out, ldo);
+    return nvs_check_launch("nvs_moe_gemm (matrix cores, LDS tiles)");
+  }
   if (dtype == NVS_BF16 && K % 8 == 0 && ldx % 8 == 0 && !g_moe_plain) {
     const dim3 grid((unsigned)(cap / tm), (unsigned)((nout + 127) / 128));
 #define NVS_MOE_CASE(MT, GLU)                                                                                                        \
@@ -365,6 +474,8 @@ extern "C" int nvs_moe_gemm(const void* X, int64_t ldx, const void* W, int dtype
                                                             (bf16_t*)out, ldo)
     if (tm == 64) {
       if (glu) NVS_MOE_CASE(4, true); else NVS_MOE_CASE(4, false);
+    } else if (tm == 128) {
+      NVS_REQUIRE(false, "nvs_moe_gemm: unreachable");
     } else {
       if (glu) NVS_MOE_CASE(1, true); else NVS_MOE_CASE(1, false);
     }

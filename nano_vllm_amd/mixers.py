@@ -347,7 +347,8 @@ class RoutedExperts(nn.Module):
         total = self.E + self.ident
         z = F.linear(xh.float(), self.router)                                     # 32-bit, [n, total (+ 1: the shared gate)]
         ids, wts = ops_seq.moe_route(z, total, self.correction, self.top, self.count, self.keep, self.scale)
-        plan = ops_seq.moe_plan(ids, self.E, 64 if n * self.top >= 64 * self.E else 16)
+        per_expert = n * self.top // self.E                 # rows an expert gets on average: the tile height follows it
+        plan = ops_seq.moe_plan(ids, self.E, 128 if per_expert >= 256 else (64 if per_expert >= 64 else 16))
         act = torch.empty(plan.cap, self.ff, dtype=xh.dtype, device=xh.device)
         ops_seq.moe_gemm(xh, self.w_gu, plan, True, act)
         rows = torch.empty(plan.cap, width, dtype=xh.dtype, device=xh.device)

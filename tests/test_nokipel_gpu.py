@@ -340,10 +340,11 @@ def moe_case(W, E, ident, ff, top, count, keep, sff, seed):
 @pytest.mark.parametrize("dtype,plain_kernel,tol", [(torch.float32, False, 2e-5), (torch.bfloat16, False, 2e-2), (torch.bfloat16, True, 2e-2)])
 @pytest.mark.parametrize("W,E,ident,ff,top,count,keep,sff,n", [(352, 7, 1, 88, 3, 2, 1, 104, 50), (40, 5, 1, 24, 2, 3, 2, 0, 33),
                                                                 (72, 4, 0, 200, 4, 1, 1, 17, 9), (64, 6, 2, 48, 2, 1, 1, 40, 700),
-                                                                (50, 3, 3, 10, 3, 2, 2, 8, 21)])
+                                                                (50, 3, 3, 10, 3, 2, 2, 8, 21), (72, 3, 1, 40, 2, 1, 1, 0, 600),
+                                                                (256, 2, 0, 160, 1, 1, 1, 0, 1100)])
 def test_routed_experts_pass_through_and_shared_expert(W, E, ident, ff, top, count, keep, sff, n, dtype, plain_kernel, tol):
     """Sizes whose inner dimensions are not multiples of the matrix-core step (or of 8: the plain kernel), few and many rows per
-    expert (both tile sizes), experts nobody chooses, pass-through experts, no shared expert."""
+    expert (all three tile sizes), experts nobody chooses, pass-through experts, no shared expert."""
     from nano_vllm_amd import ops_seq
     from nano_vllm_amd.mixers import RoutedExperts
     cfg, p = moe_case(W, E, ident, ff, top, count, keep, sff, seed=W + n)
