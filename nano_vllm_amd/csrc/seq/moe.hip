@@ -290,21 +290,20 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(const bf16_t* __rest
 }
 
 // LDS-tiled matrix-core form for steps with many rows per expert (tiles of 128 rows). A workgroup of four wavefronts computes
-// 128 rows x 128 features (GLU: gate and up of the same 128 features, 256 weight rows) in steps of 32 along k: all threads
-// load the step's operands with 16-byte loads — the NEXT step's loads are issued before the current step is computed — into
-// LDS as [row][32 + 8]; a wavefront owns 64 rows x 64 features (4 x 4 MFMA tiles per operand set) and reads its operands as
-// 16-byte LDS reads: 8 (12) reads for 16 (32) MFMAs. The grid is one-dimensional and XCD-aware: workgroups are dealt to the
-// eight XCDs round-robin, so workgroup id -> (id % 8) * per_xcd + id / 8 gives every XCD a CONTIGUOUS run of tiles, ordered
-// feature tile major / row tile minor: consecutive tiles of an XCD share a weight tile (all row tiles of one expert), which
-// its L2 then serves.
+// 128 rows x 128 features (GLU: gate and up of the same 64 features; 128 weight rows either way) in steps of 64 along k: all
+// threads load the step's operands with 16-byte loads — the NEXT step's loads are issued before the current step is computed —
+// into LDS as [row][64 + 8]; a wavefront owns 64 rows x 64 weight rows (4 x 4 MFMA tiles) and reads its operands as 16-byte LDS
+// reads: 16 reads for 32 MFMAs per step. The grid is one-dimensional and XCD-aware: workgroups are dealt to the eight XCDs
+// round-robin, so workgroup id -> (id % 8) * per_xcd + id / 8 gives every XCD a CONTIGUOUS run of tiles, ordered feature tile
+// major / row tile minor: consecutive tiles of an XCD share a weight tile (all row tiles of one expert), which its L2 then serves.
 template <bool GLU>
 __global__ __launch_bounds__(256) void moe_gemm_tiled_kernel(const bf16_t* __restrict__ X, int64_t ldx, const bf16_t* __restrict__ W, int nout,
                                                              int K, const int32_t* __restrict__ tile_expert,
                                                              const int32_t* __restrict__ row_token, int tiles_m, int tiles_n,
                                                              bf16_t* __restrict__ out, int64_t ldo) {
-  constexpr int BM = 128, BN = 128, BK = 32, LDK = BK + 8, NG = GLU ? 2 : 1;
+  constexpr int BM = 128, BW = 128, BK = 64, LDK = BK + 8, NG = GLU ? 2 : 1, FB = 4 / NG, BN = BW / NG;   // BN features per tile
   __shared__ __attribute__((aligned(16))) bf16_t Xs[BM][LDK];
-  __shared__ __attribute__((aligned(16))) bf16_t Ws[NG * BN][LDK];
+  __shared__ __attribute__((aligned(16))) bf16_t Ws[BW][LDK];      // GLU: rows [0, 64) gate, [64, 128) up of the tile's features
   const int per_xcd = gridDim.x / 8;
   const int logical = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
   if (logical >= tiles_m * tiles_n) return;
@@ -315,70 +314,72 @@ __global__ __launch_bounds__(256) void moe_gemm_tiled_kernel(const bf16_t* __res
   const int wm = wave & 1, wn = wave >> 1;
   const int64_t row0 = (int64_t)rt * BM;
   const bf16_t* We = W + (int64_t)e * NG * nout * K;
-  // staging: unit u = tid + 256 i -> (row u >> 2, 8 elements of k at (u & 3) * 8)
-  const int sk = (tid & 3) * 8;
-  const bf16_t* xsrc[2];
-  const bf16_t* wsrc[2 * NG];
+  // staging: unit u = tid + 256 i -> (row u >> 3, 8 elements of k at (u & 7) * 8); four units of each operand per thread
+  const int sk = (tid & 7) * 8, sr = tid >> 3;
+  const bf16_t* xsrc[4];
+  const bf16_t* wsrc[4];
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const int r = (tid >> 2) + 64 * i;
+  for (int i = 0; i < 4; ++i) {
+    const int r = sr + 32 * i;
     const int tok = row_token[row0 + r];
     xsrc[i] = tok >= 0 ? X + (GLU ? (int64_t)tok : row0 + r) * ldx + sk : nullptr;
-  }
-#pragma unroll
-  for (int i = 0; i < 2 * NG; ++i) {
-    const int r = (tid >> 2) + 64 * i, g = r / BN, f = ft * BN + r % BN;
+    const int g = r / BN, f = ft * BN + r % BN;
     wsrc[i] = f < nout ? We + ((int64_t)g * nout + f) * K + sk : nullptr;
   }
   const u32x4_t zero4 = u32x4_t{0u, 0u, 0u, 0u};
-  u32x4_t xr[2], wr[2 * NG];
+  u32x4_t xr[4], wr[4];
   auto fetch = [&](int k0) {
     const bool kin = k0 + sk < K;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) xr[i] = (kin && xsrc[i]) ? *(const u32x4_t*)(xsrc[i] + k0) : zero4;
+    for (int i = 0; i < 4; ++i) xr[i] = (kin && xsrc[i]) ? *(const u32x4_t*)(xsrc[i] + k0) : zero4;
 #pragma unroll
-    for (int i = 0; i < 2 * NG; ++i) wr[i] = (kin && wsrc[i]) ? *(const u32x4_t*)(wsrc[i] + k0) : zero4;
+    for (int i = 0; i < 4; ++i) wr[i] = (kin && wsrc[i]) ? *(const u32x4_t*)(wsrc[i] + k0) : zero4;
   };
-  f32x4_t acc[NG][4][4];
+  // accumulators: weight-row block wb of this wavefront's 64 weight rows x row block rb. GLU: a wavefront's 64 weight rows are
+  // 32 gate rows and the 32 up rows of the SAME features (wb 0, 1 gate; 2, 3 up), so the activation needs no exchange.
+  f32x4_t acc[4][4];
 #pragma unroll
-  for (int g = 0; g < NG; ++g)
+  for (int wb = 0; wb < 4; ++wb)
 #pragma unroll
-    for (int fb = 0; fb < 4; ++fb)
+    for (int rb = 0; rb < 4; ++rb) acc[wb][rb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  int wrow[4];                                      // LDS row of this lane's operand for weight-row block wb
 #pragma unroll
-      for (int rb = 0; rb < 4; ++rb) acc[g][fb][rb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  for (int wb = 0; wb < 4; ++wb) wrow[wb] = GLU ? (wb / FB) * BN + wn * 32 + (wb % FB) * 16 + li : wn * 64 + wb * 16 + li;
   fetch(0);
   for (int k0 = 0; k0 < K; k0 += BK) {
     __syncthreads();                                // the previous step's readers are done
 #pragma unroll
-    for (int i = 0; i < 2; ++i) *(u32x4_t*)&Xs[(tid >> 2) + 64 * i][sk] = xr[i];
-#pragma unroll
-    for (int i = 0; i < 2 * NG; ++i) *(u32x4_t*)&Ws[(tid >> 2) + 64 * i][sk] = wr[i];
+    for (int i = 0; i < 4; ++i) {
+      *(u32x4_t*)&Xs[sr + 32 * i][sk] = xr[i];
+      *(u32x4_t*)&Ws[sr + 32 * i][sk] = wr[i];
+    }
     __syncthreads();
     if (k0 + BK < K) fetch(k0 + BK);
-    bf16x8_t xb[4];
 #pragma unroll
-    for (int rb = 0; rb < 4; ++rb) xb[rb] = *(const bf16x8_t*)&Xs[wm * 64 + rb * 16 + li][lk];
+    for (int kk = 0; kk < BK; kk += 32) {
+      bf16x8_t xb[4];
 #pragma unroll
-    for (int g = 0; g < NG; ++g)
+      for (int rb = 0; rb < 4; ++rb) xb[rb] = *(const bf16x8_t*)&Xs[wm * 64 + rb * 16 + li][kk + lk];
 #pragma unroll
-      for (int fb = 0; fb < 4; ++fb) {
-        const bf16x8_t wa = *(const bf16x8_t*)&Ws[g * BN + wn * 64 + fb * 16 + li][lk];
+      for (int wb = 0; wb < 4; ++wb) {
+        const bf16x8_t wa = *(const bf16x8_t*)&Ws[wrow[wb]][kk + lk];
 #pragma unroll
-        for (int rb = 0; rb < 4; ++rb) acc[g][fb][rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa, xb[rb], acc[g][fb][rb], 0, 0, 0);
+        for (int rb = 0; rb < 4; ++rb) acc[wb][rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa, xb[rb], acc[wb][rb], 0, 0, 0);
       }
+    }
   }
-  // lane: row li of row block rb, features 16 fb + 4 (lane >> 4) + 0..3 of its wavefront's 64
+  // lane: row li of row block rb; features 16 fb + 4 (lane >> 4) + 0..3 of its wavefront's 64 (GLU: 32)
 #pragma unroll
   for (int rb = 0; rb < 4; ++rb) {
     const int64_t r = row0 + wm * 64 + rb * 16 + li;
     if (row_token[r] < 0) continue;
 #pragma unroll
-    for (int fb = 0; fb < 4; ++fb) {
-      const int f = ft * BN + wn * 64 + fb * 16 + (lane >> 4) * 4;
+    for (int fb = 0; fb < FB; ++fb) {
+      const int f = ft * BN + wn * (16 * FB) + fb * 16 + (lane >> 4) * 4;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         if (f + i < nout) {
-          const float v = GLU ? glu_value(acc[0][fb][rb][i], acc[NG - 1][fb][rb][i], 0, 0.f, 0.f) : acc[0][fb][rb][i];
+          const float v = GLU ? glu_value(acc[fb][rb][i], acc[GLU ? fb + FB : fb][rb][i], 0, 0.f, 0.f) : acc[fb][rb][i];
           out[r * ldo + f + i] = (bf16_t)v;
         }
       }
@@ -456,7 +457,8 @@ extern "C" int nvs_moe_gemm(const void* X, int64_t ldx, const void* W, int dtype
   if (cap == 0) return NVS_OK;
   hipStream_t st = (hipStream_t)stream;
   if (dtype == NVS_BF16 && K % 8 == 0 && ldx % 8 == 0 && !g_moe_plain && tm == 128) {
-    const int tiles_m = (int)(cap / 128), tiles_n = (nout + 127) / 128;
+    const int bn = glu ? 64 : 128;                  // features per tile
+    const int tiles_m = (int)(cap / 128), tiles_n = (nout + bn - 1) / bn;
     const int64_t blocks = ((int64_t)tiles_m * tiles_n + 7) / 8 * 8;
     NVS_REQUIRE(blocks < (1ll << 31), "nvs_moe_gemm: step too large");
     if (glu)
