@@ -114,28 +114,40 @@ __global__ void xielu_kernel(const T* __restrict__ in, const T* __restrict__ pq,
 
 // Input-side ("pre") norm on the 32-bit residual: x[t] += a[t] + b[t] first (either may be absent), then every one of
 // `groups` equal parts of the row is divided by its own root mean square and the row is multiplied by w. One workgroup per
-// row, one wavefront per group at a time. With `rows` the kernel only reads: out[r] = norm(x[rows[r]]).
+// row; a group is served by one wavefront (several groups per wavefront, in turn, when there are more groups than wavefronts)
+// or by `blockDim / 64 / groups` wavefronts together when there are fewer. With `rows` the kernel only reads:
+// out[r] = norm(x[rows[r]]).
 template <typename T>
 __global__ void add_group_norm_kernel(float* __restrict__ x, const T* __restrict__ a, const float* __restrict__ b,
                                       const int32_t* __restrict__ rows, const T* __restrict__ w, int width, int groups, float eps,
                                       T* __restrict__ out) {
+  __shared__ float red[16];
   const int64_t r = blockIdx.x;
   const int64_t t = rows ? (int64_t)rows[r] : r;
   const int gsz = width / groups, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
   float* xr = x + t * width;
-  for (int g = wave; g < groups; g += nw) {
+  const int wpg = nw > groups ? nw / groups : 1;    // wavefronts per group (the host makes nw a multiple of groups then)
+  const int first = wave / wpg, step = nw / wpg, idx = (wave % wpg) * 64 + lane, stride = wpg * 64;
+  for (int g = first; g < groups; g += step) {
     const int c0 = g * gsz;
     float ss = 0.f;
-    for (int c = lane; c < gsz; c += 64) {
+    for (int c = idx; c < gsz; c += stride) {
       float v = xr[c0 + c];
       if (a) v += ldf(a + t * width + c0 + c);
       if (b) v += b[t * width + c0 + c];
       if (a || b) xr[c0 + c] = v;
       ss += v * v;
     }
-    if (!out) continue;
-    const float k = 1.f / sqrtf(wave_sum(ss) / (float)gsz + eps);
-    for (int c = lane; c < gsz; c += 64) stf(out + r * width + c0 + c, xr[c0 + c] * k * ldf(w + c0 + c));   // (this lane wrote xr[c0 + c])
+    if (!out) continue;                             // (uniform over the workgroup)
+    ss = wave_sum(ss);
+    if (wpg > 1) {                                  // (then every wavefront runs this loop exactly once)
+      if (lane == 0) red[wave] = ss;
+      __syncthreads();
+      ss = 0.f;
+      for (int i = 0; i < wpg; ++i) ss += red[first * wpg + i];
+    }
+    const float k = 1.f / sqrtf(ss / (float)gsz + eps);
+    for (int c = idx; c < gsz; c += stride) stf(out + r * width + c0 + c, xr[c0 + c] * k * ldf(w + c0 + c));   // (this thread wrote xr[c0 + c])
   }
 }
 
@@ -186,7 +198,9 @@ extern "C" int nvs_add_group_norm(float* x, const void* a, const float* b, const
               width, groups);
   NVS_REQUIRE(!rows || (!a && !b), "nvs_add_group_norm: selected rows are only read");
   if (nrows == 0) return NVS_OK;
-  const int threads = 64 * (groups < 4 ? groups : 4);      // a wavefront per group, four groups at a time
+  // a wavefront per group, four groups at a time; wide groups that are fewer than four are shared by 4 / groups wavefronts
+  int threads = 64 * (groups < 4 ? groups : 4);
+  if (groups < 4 && 4 % groups == 0 && width / groups >= 512) threads = 256;
   NVS_DISPATCH(dtype, add_group_norm_kernel<T><<<dim3((unsigned)nrows), dim3(threads), 0, (hipStream_t)stream>>>(
                           x, (const T*)a, b, rows, (const T*)w, width, groups, eps, (T*)out));
   return nvs_check_launch("nvs_add_group_norm");
