@@ -78,7 +78,10 @@ def _mixer(width: int, spec: dict, eps: float, block_size: int):
         return AttentionMixer(width, m["heads"], m.get("kv_heads", m["heads"]), m["dim"], m.get("vdim", m["dim"]), m["scale"], eps,
                               block_size, chunk=int(mask["size"]) if mask else 0, rot_dims=int(rot["dims"]) if rot else 0,
                               rot_base=float(rot["base"]) if rot else 10000.0)
-    return LightningMixer(width, m["heads"], m["dim"], m.get("vdim", m["dim"]), m["decay"], eps)
+    decay = m["decay"]
+    if isinstance(decay, (int, float)):                # one number: every head decays alike
+        decay = [decay] * m["heads"]
+    return LightningMixer(width, m["heads"], m["dim"], m.get("vdim", m["dim"]), decay, eps)
 
 
 def _feed_forward(width: int, mlp: dict | None):

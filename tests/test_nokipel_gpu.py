@@ -440,7 +440,8 @@ def engine(path, dtype="float32", pages=40, page=16, live=4, **kw):
     from nano_vllm_amd import LLM
     kw.setdefault("enforce_eager", True)
     kw.setdefault("max_num_batched_tokens", 1024)
-    return LLM(path, dtype=dtype, kvcache_block_size=page, num_kvcache_blocks=pages, max_num_seqs=live, max_model_len=640, **kw)
+    kw.setdefault("max_model_len", 640)
+    return LLM(path, dtype=dtype, kvcache_block_size=page, num_kvcache_blocks=pages, max_num_seqs=live, **kw)
 
 
 def rel(got, want, scale):
@@ -573,6 +574,34 @@ def test_greedy_generation_through_generate_matches_the_plain_model(checkpoints,
                 assert t == int(top.indices[0])
                 checked += 1
     assert checked >= 30
+
+
+def test_sampled_generation_is_reproducible_and_preemption_recomputes_pages_and_state(checkpoints):
+    """A pool so small that running sequences are preempted: a preempted sequence loses its pages AND its state slot (every
+    run of a repeated layer included) and is recomputed from its first token; greedy results must not change, and a sampled
+    run repeats itself."""
+    from nano_vllm_amd import SamplingParams
+    path = checkpoints["float32"][0]
+    g = torch.Generator().manual_seed(2)
+    prompts = [torch.randint(0, 200, (n,), generator=g).tolist() for n in (30, 31, 29, 17)]
+    greedy = SamplingParams(temperature=0.0, max_tokens=40, ignore_eos=True)
+    outs = []
+    for pages in (40, 11):
+        llm = engine(path, "float32", pages=pages, max_num_batched_tokens=256, max_model_len=128)
+        try:
+            outs.append([o["token_ids"] for o in llm.generate(prompts, greedy, use_tqdm=False)])
+        finally:
+            llm.exit()
+    assert outs[0] == outs[1]
+    warm = []
+    for _ in range(2):
+        llm = engine(path, "bfloat16", pages=40, max_num_batched_tokens=256, max_model_len=128)
+        try:
+            warm.append([o["token_ids"] for o in llm.generate(prompts, SamplingParams(temperature=0.8, max_tokens=16, ignore_eos=True),
+                                                               use_tqdm=False)])
+        finally:
+            llm.exit()
+    assert warm[0] == warm[1] and warm[0] != [o[:16] for o in outs[0]]
 
 
 def test_the_schedule_replayer_as_a_program(checkpoints, tmp_path):
