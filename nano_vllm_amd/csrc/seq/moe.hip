@@ -456,7 +456,8 @@ extern "C" int nvs_moe_gemm(const void* X, int64_t ldx, const void* W, int dtype
               "nvs_moe_gemm: %d x %d, %lld rows in tiles of %d", nout, K, (long long)cap, tm);
   if (cap == 0) return NVS_OK;
   hipStream_t st = (hipStream_t)stream;
-  if (dtype == NVS_BF16 && K % 8 == 0 && ldx % 8 == 0 && !g_moe_plain && tm == 128) {
+  const bool matrix_cores = dtype == NVS_BF16 && K % 8 == 0 && ldx % 8 == 0 && !g_moe_plain;
+  if (matrix_cores && tm == 128) {
     const int bn = glu ? 64 : 128;                  // features per tile
     const int tiles_m = (int)(cap / 128), tiles_n = (nout + bn - 1) / bn;
     const int64_t blocks = ((int64_t)tiles_m * tiles_n + 7) / 8 * 8;
@@ -469,15 +470,13 @@ extern "C" int nvs_moe_gemm(const void* X, int64_t ldx, const void* W, int dtype
                                                                                  row_token, tiles_m, tiles_n, (bf16_t*)out, ldo);
     return nvs_check_launch("nvs_moe_gemm (matrix cores, LDS tiles)");
   }
-  if (dtype == NVS_BF16 && K % 8 == 0 && ldx % 8 == 0 && !g_moe_plain) {
+  if (matrix_cores) {
     const dim3 grid((unsigned)(cap / tm), (unsigned)((nout + 127) / 128));
 #define NVS_MOE_CASE(MT, GLU)                                                                                                        \
   moe_gemm_mfma_kernel<MT, GLU><<<grid, dim3(256), 0, st>>>((const bf16_t*)X, ldx, (const bf16_t*)W, nout, K, tile_expert, row_token,  \
                                                             (bf16_t*)out, ldo)
     if (tm == 64) {
       if (glu) NVS_MOE_CASE(4, true); else NVS_MOE_CASE(4, false);
-    } else if (tm == 128) {
-      NVS_REQUIRE(false, "nvs_moe_gemm: unreachable");
     } else {
       if (glu) NVS_MOE_CASE(1, true); else NVS_MOE_CASE(1, false);
     }
